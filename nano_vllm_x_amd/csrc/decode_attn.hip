@@ -486,7 +486,7 @@ __device__ __forceinline__ unsigned dec_lds_addr(const void* p) {
 }
 // 64 lanes x 16 bytes from per-lane global addresses to 1 KB of LDS starting at a wave-uniform address, as a streaming
 // (non-temporal) read.  Issued from inline assembly: the compiler's own LDS-DMA builtin makes every later LDS read wait
-// for the copy.  m0 has no other user in this kernel: the toolchain refuses m0 in a clobber list (reserved register), so tests/test_abi_exports.py disassembles the library and checks that every access to m0 is one of these moves.
+// for the copy.  m0 has no other user in this kernel (the toolchain refuses m0 in a clobber list: it is a reserved register).
 __device__ __forceinline__ void dec_dma16(const char* g, unsigned lds_addr) {
     const unsigned uni = (unsigned)__builtin_amdgcn_readfirstlane((int)lds_addr);
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt" : : "v"(g), "s"(uni) : "memory");
