@@ -40,8 +40,10 @@ typedef void* nvx_stream_t;
  * Bump it whenever a signature below changes.
  *   2: nvx_decode_step_setup gained `prev_ids`.
  *   3: float16 entry points (`*_f16`) added.
- *   4: direct-peer all-reduce (`nvx_peer_*`) and sharded sampling (`nvx_sample_shard`, `nvx_sample_pick`) added. */
-#define NVX_ABI_VERSION 7
+ *   4: direct-peer all-reduce (`nvx_peer_*`) and sharded sampling (`nvx_sample_shard`, `nvx_sample_pick`) added.
+ *   8: layers with a 32-bit residual stream and per-sequence state (`nvx_boundary_norm`, `nvx_canon_conv`, `nvx_relu2`,
+ *      `nvx_mingru_scan`) and latent attention (`nvx_latent_prep`, `nvx_latent_attn`) added. */
+#define NVX_ABI_VERSION 8
 
 /* Library identification and diagnostics. */
 int nvx_abi_version(void);
@@ -441,6 +443,50 @@ int nvx_lmhead_sample_f16(const void* w_packed, int64_t n_rows, int64_t k, const
                           int64_t batch, const float* temperatures, int64_t vocab_offset, int64_t vocab,
                           uint64_t seed, uint64_t offset, void* ws, int64_t ws_bytes, uint64_t* key_out,
                           int64_t* out_ids, void* logits_out, int64_t logits_row_stride, nvx_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Layer stacks with a float32 residual stream, per-sequence recurrent state and latent attention.
+ * One entry point serves every activation format: `fmt` 0 = bfloat16, 1 = float16, 2 = float32 (what the
+ * matrix products read and write).  Norm weights, taps, mixing weights, the stream and all state are float32.
+ * A batch is ragged: tokens [qo_indptr[b], qo_indptr[b+1]) belong to sequence b, tok_seq[t] = b for each of them;
+ * pos0[b] is the position of its first token in this step and state_slot[b] its slot in the state tensors (a
+ * negative slot marks a padding row: nothing of it is read or written).  With qo_indptr == NULL every sequence has
+ * exactly one token (a decode step).  A sequence at position 0 takes zeros for its state instead of reading it.
+ *
+ * nvx_boundary_norm, per token t:
+ *     r = res[t] + m[t] / sqrt(mean(m[t]^2) + eps) * (1 + w_post)        (res == NULL: the normed m alone)
+ *     hist[hist_slot][t] = r                                             (hist_slot >= 0; slots hist_stride floats apart)
+ *     x = sum_{j < n_mix} mix[j] * hist[j][t]   (n_mix > 0; hist_slot < n_mix is r itself)   else x = r
+ *     x_out[t] = x;   w_pre != NULL:  y = x / sqrt(mean(x^2) + eps) * (1 + w_pre)  ->  y_f32 or y_act (exactly one)
+ * nvx_canon_conv:  out[t] = h[t] + sum_j taps[:, j] * h[t - (taps_n - 1) + j]  over the tokens of t's own sequence;
+ *     inputs before this step come from state[slot] (taps_n - 1 rows of `width`, oldest first), which is then
+ *     replaced by the sequence's last taps_n - 1 inputs.
+ * nvx_relu2:  y = max(x, 0)^2, element by element.
+ * nvx_mingru_scan:  zxg[t] = [z | u | g] pre-activations, `width` each, rows row_stride elements apart;
+ *     S <- (1 - sigmoid(z)) S + sigmoid(z) * (u >= 0 ? u + 1/2 : sigmoid(u));  out[t] = S * g * sigmoid(g);
+ *     S starts from state[slot] (float32, `width`) and the sequence's last S is written back.
+ * nvx_latent_prep:  x[t] = [query latent (q_rank) | key/value latent (kv_rank) | gate pre-activation per head];
+ *     cq[t] = RMS-normed query latent * w_q;  cache[slots[t]] = RMS-normed key/value latent * w_kv (negative slot:
+ *     skipped);  gate[t][h] = sigmoid(.) in float32.
+ * nvx_latent_attn:  q, out: (heads, n_tok, rank) in the activation format, cache: (slots, rank).  Token t of sequence b
+ *     attends over the latents at slots kv_indices[kv_start[b] + j], j <= kv_len[b] - q_len[b] + (t - qo_indptr[b]):
+ *     out[h][t] = gate[t][h] * sum_j softmax_j(scale * q[h][t] . c_j) c_j   (gate may be NULL).  rank <= 1024. */
+int nvx_boundary_norm(const void* m, int64_t m_row_stride, int fmt, const float* res, const float* w_post, float* hist,
+                      int64_t hist_stride, int hist_slot, int n_mix, const float* mix, float* x_out, const float* w_pre,
+                      float* y_f32, void* y_act, int64_t n_tok, int64_t width, float eps, nvx_stream_t stream);
+int nvx_canon_conv(const float* h, const float* taps, int taps_n, float* state, int64_t n_slots, const int32_t* tok_seq,
+                   const int32_t* qo_indptr, const int64_t* pos0, const int32_t* state_slot, void* out, int fmt,
+                   int64_t n_tok, int64_t n_seq, int64_t width, nvx_stream_t stream);
+int nvx_relu2(const void* x, void* y, int fmt, int64_t n, nvx_stream_t stream);
+int nvx_mingru_scan(const void* zxg, int64_t row_stride, int fmt, float* state, int64_t n_slots, const int32_t* qo_indptr,
+                    const int64_t* pos0, const int32_t* state_slot, void* out, int64_t n_tok, int64_t n_seq, int64_t width,
+                    nvx_stream_t stream);
+int nvx_latent_prep(const void* x, int64_t x_row_stride, int fmt, const float* w_q, const float* w_kv, float eps,
+                    const int64_t* slots, void* cq, void* cache, int64_t n_slots, float* gate, int64_t n_tok, int64_t q_rank,
+                    int64_t kv_rank, int64_t heads, nvx_stream_t stream);
+int nvx_latent_attn(const void* q, const void* cache, int fmt, const int32_t* kv_indices, const int64_t* kv_start,
+                    const int32_t* kv_len, const int32_t* qo_indptr, const int32_t* tok_seq, const float* gate, void* out,
+                    int64_t heads, int64_t rank, int64_t n_tok, float scale, nvx_stream_t stream);
 
 #ifdef __cplusplus
 }

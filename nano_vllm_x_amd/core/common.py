@@ -57,6 +57,7 @@ class Sequence:
     # plain class attributes (not dataclass fields), set per object where they apply
     partial_of = None      # chunked prefill: the sequence this truncated copy stands for
     length_limit = None    # engine cache: total length at which a LENGTH stop rule fires (0 = none)
+    state_slot = None      # models with per-sequence state: the sequence's slot in the state tensors while it runs
 
     @property
     def num_new_tokens(self) -> int:
@@ -69,6 +70,8 @@ class ForwardBatch:
     forward_mode: ForwardMode
     num_seqs: int
     seqs: list
+    # rows of the step's flat token list whose hidden states (and logits) are asked for; None: each sequence's last token
+    want_rows: Optional[list] = None
 
 
 @dataclass

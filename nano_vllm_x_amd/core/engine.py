@@ -19,8 +19,10 @@ from .scheduler import Scheduler
 
 class EngineCore:
     def __init__(self, kv_cache_size: int, max_bs: int, context_len: int = 2048, prefix_reuse: bool = False,
-                 max_prefill_tokens: Optional[int] = None, stop_at_context_len: bool = False, chunked_prefill: bool = False):
+                 max_prefill_tokens: Optional[int] = None, stop_at_context_len: bool = False, chunked_prefill: bool = False,
+                 state_slots: Optional[int] = None):
         self.context_len = context_len
+        self.state_slots = state_slots
         self.prefix_reuse = prefix_reuse
         self.max_prefill_tokens = max_prefill_tokens
         # The reference has no stop rule tied to the context length: a request without max_tokens and with
@@ -29,7 +31,7 @@ class EngineCore:
         self.stop_at_context_len = stop_at_context_len
         self.chunked_prefill = chunked_prefill
         self.scheduler = Scheduler(kv_cache_size=kv_cache_size, max_bs=max_bs, prefix_reuse=prefix_reuse,
-                                   max_prefill_tokens=max_prefill_tokens, chunked_prefill=chunked_prefill)
+                                   max_prefill_tokens=max_prefill_tokens, chunked_prefill=chunked_prefill, state_slots=state_slots)
 
     def add_sequence(self, sequence_id: str, prompt_token_ids: list, sampling_params: SamplingParams):
         if len(prompt_token_ids) > self.context_len:   # keep the tail (engine.py:59-60)
@@ -40,6 +42,16 @@ class EngineCore:
         sampling_params = replace(sampling_params)
         self.scheduler.add_sequence(Sequence(seq_id=sequence_id, token_ids=prompt_token_ids, num_tokens=n,
                                              prompt_len=n, sampling_params=sampling_params))
+
+    def extend_sequence(self, sequence_id: str, token_ids: list):
+        """More tokens for a sequence whose input arrives in pieces: they join the tokens that wait to be computed."""
+        seq = self.scheduler.get_sequence(sequence_id)
+        if seq is None:
+            raise KeyError(sequence_id)
+        if len(seq.token_ids) + len(token_ids) > self.context_len:
+            raise ValueError(f"sequence {sequence_id!r} would grow beyond the context length {self.context_len}")
+        seq.token_ids.extend(token_ids)
+        seq.num_tokens = seq.prompt_len = len(seq.token_ids)
 
     def abort_sequence(self, sequence_id: str):
         seq = self.scheduler.get_sequence(sequence_id)
@@ -125,7 +137,7 @@ class Engine(EngineCore):
                  nccl_port: int = 29500, device_ids: Optional[list] = None, enforce_eager: bool = False,
                  context_len: int = 2048, kv_cache_size: Optional[int] = None, seed: int = 0, prefix_reuse: bool = False,
                  max_prefill_tokens: Optional[int] = None, stop_at_context_len: bool = False, chunked_prefill: bool = False,
-                 run_ahead: bool = False):
+                 run_ahead: bool = False, dtype: Optional[str] = None):
         from .model_runner import ModelRunner
 
         # pp_size > 1: every rank runs this same engine and scheduler.  Time advances in ticks: at tick t
@@ -134,7 +146,7 @@ class Engine(EngineCore):
         # pp_size batches in flight, as engine.py:102-117 keeps them
         self.model_runner = ModelRunner(model=model, max_bs=max_bs, tp_size=tp_size, nccl_port=nccl_port,
                                         device_ids=device_ids, enforce_eager=enforce_eager, context_len=context_len,
-                                        seed=seed, pp_size=pp_size)
+                                        seed=seed, pp_size=pp_size, dtype=dtype)
         self.model_runner.load_model()
         if kv_cache_size is None:
             kv_cache_size = self.model_runner.profile_kv_cache_size(gpu_memory_utilization)
@@ -142,7 +154,7 @@ class Engine(EngineCore):
         self.model_runner.initialize_kv_cache(kv_cache_size)
         super().__init__(kv_cache_size=kv_cache_size, max_bs=max_bs, context_len=context_len, prefix_reuse=prefix_reuse,
                          max_prefill_tokens=max_prefill_tokens, stop_at_context_len=stop_at_context_len,
-                         chunked_prefill=chunked_prefill)
+                         chunked_prefill=chunked_prefill, state_slots=self.model_runner.state_slots)
         self.scheduler.on_release = self.model_runner.release_sequence
         self._inflight = None
         # run_ahead: step_overlapped() queues decode step N+1 behind step N before N's ids have reached the
@@ -157,6 +169,27 @@ class Engine(EngineCore):
         self._pp_window: deque = deque(maxlen=max(pp_size, 1))   # the batches of the last pp_size ticks, newest last
         self._pp_aborts: list = []
         self.pp_stats = {"ticks": 0, "stage_busy_ticks": 0}
+
+    def run_given(self, plan, want=None):
+        """One step whose content is given (Scheduler.schedule_given): `plan` lists (seq_id, n) pairs; `want`, for each
+        entry, the places among its n tokens whose logits are returned (default: none).  Runs the batch through the model
+        runner's own step, samples nothing, and returns the logits (wanted rows in order, vocab) -- None if nothing is wanted."""
+        if self._inflight is not None or self._ahead is not None:
+            raise RuntimeError("a sampled step is in flight")
+        batch = self.scheduler.schedule_given(plan)
+        if batch is None:
+            return None
+        rows, base = [], 0
+        for (_, n), places in zip(plan, want or [[] for _ in plan]):
+            for k in places:
+                if not 0 <= k < n:
+                    raise ValueError(f"wanted place {k} outside the {n} tokens of its entry")
+                rows.append(base + k)
+            base += n
+        batch.want_rows = rows
+        logits = self.model_runner.compute_logits(batch)
+        self.scheduler.commit_given(batch)
+        return logits if rows else None
 
     def step(self) -> list:
         if self._inflight is None and not self.begin_step():
@@ -322,7 +355,8 @@ class Engine(EngineCore):
             self.model_runner.block_table.release(seq_id)
         self.model_runner._sp_key = None
         self.scheduler = Scheduler(kv_cache_size=self.kv_cache_size, max_bs=self.scheduler.max_bs, prefix_reuse=self.prefix_reuse,
-                                   max_prefill_tokens=self.max_prefill_tokens, chunked_prefill=self.chunked_prefill)
+                                   max_prefill_tokens=self.max_prefill_tokens, chunked_prefill=self.chunked_prefill,
+                                   state_slots=self.state_slots)
         self.scheduler.on_release = self.model_runner.release_sequence
 
     def wait_until_ready(self):

@@ -55,6 +55,76 @@ class KVCachePool:
         store_kvcache(k_cache, v_cache, self.k_cache[i], self.v_cache[i], index)
 
 
+class LatentCachePool:
+    """Cache of layers that keep ONE latent vector per token (latent attention): per such layer a tensor
+    (tokens, rank) in the activations' format.  Slot ids are the same token slots the allocator below hands out, so a
+    sequence's slot list serves every layer, whatever its rank."""
+
+    def __init__(self, dtype: torch.dtype, device: torch.device, num_tokens: int, ranks: dict):
+        self.dtype, self.device, self.num_tokens = dtype, device, num_tokens
+        # zero-filled for the same reason as the K/V pool: a masked key must not bring NaN from stale memory
+        self.latents = {layer: torch.zeros((num_tokens, rank), dtype=dtype, device=device) for layer, rank in ranks.items()}
+
+    def get(self, layer: int) -> torch.Tensor:
+        return self.latents[layer]
+
+    @staticmethod
+    def bytes_per_token(ranks: dict, dtype: torch.dtype) -> int:
+        return sum(ranks.values()) * dtype.itemsize
+
+
+class RecurrentStatePool:
+    """Per-sequence state of layers that carry something from token to token: float32 tensors whose first index is a
+    state slot.  `shapes`: name -> shape of one slot's entry.  One slot more than asked for is allocated: the last
+    one is where padding rows of a captured step may point.  Nothing is cleared when a slot changes hands: a sequence
+    that starts at position 0 does not read its state (the kernels take zeros), and writes it at the end of its first step."""
+
+    def __init__(self, device: torch.device, num_slots: int, shapes: dict):
+        self.device, self.num_slots = device, num_slots
+        self.tensors = {name: torch.zeros((num_slots + 1,) + tuple(shape), dtype=torch.float32, device=device)
+                        for name, shape in shapes.items()}
+
+    def get(self, name) -> torch.Tensor:
+        return self.tensors[name]
+
+    @staticmethod
+    def bytes_per_slot(shapes: dict) -> int:
+        total = 0
+        for shape in shapes.values():
+            n = 4
+            for d in shape:
+                n *= d
+            total += n
+        return total
+
+
+class StateSlotAllocator:
+    """Free list of state slots (host side): lowest free slot first, so a trace of admissions is reproducible."""
+
+    def __init__(self, size: int):
+        self.size = size
+        self._free: list = list(range(size))
+        heapq.heapify(self._free)
+        self.owner: dict = {}      # seq_id -> slot
+
+    def num_free(self) -> int:
+        return len(self._free)
+
+    def alloc(self, seq_id: str) -> Optional[int]:
+        if seq_id in self.owner:
+            return self.owner[seq_id]
+        if not self._free:
+            return None
+        slot = heapq.heappop(self._free)
+        self.owner[seq_id] = slot
+        return slot
+
+    def free(self, seq_id: str):
+        slot = self.owner.pop(seq_id, None)
+        if slot is not None:
+            heapq.heappush(self._free, slot)
+
+
 class KVCacheAllocator:
     """Stack of free token slots (kv_cache.py:101-117): a fresh pool hands out 0, 1, 2, ...; freed
     slots are reissued last-in first-out.

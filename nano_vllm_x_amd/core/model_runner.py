@@ -26,7 +26,9 @@ from .. import distributed as tpd
 from .. import ops
 from ..layers.attention import AttentionBackend, AttentionMetadata, BlockTable, PagedDecodeWrapper, attention_kv_cache
 from ..layers.sampler import Sampler
-from ..qwen3 import Qwen3Config, Qwen3ForCausalLM, load_config
+from ..layers.seq_state import SeqStateBackend, SeqStateCache
+from ..qwen3 import Qwen3Config
+from ..registry import load_config, model_class_of
 from .common import ForwardBatch, ForwardMode
 from .hip_graph import HIPGraph, decode_batch_ladder
 from .kv_cache import KVCachePool
@@ -49,7 +51,7 @@ def get_model_config_per_gpu(cfg: Qwen3Config, tp_size: int):
 class ModelRunner:
     def __init__(self, model: str, max_bs: int, tp_size: int = 1, nccl_port: int = 29500,
                  device_ids: Optional[list] = None, enforce_eager: bool = False, context_len: int = 2048,
-                 seed: int = 0, config: Optional[Qwen3Config] = None, pp_size: int = 1):
+                 seed: int = 0, config=None, pp_size: int = 1, dtype: Optional[str] = None):
         if not torch.cuda.is_available():
             raise RuntimeError("ModelRunner needs an MI355X: the HIP path has no CPU fallback")
         self.model_path, self.max_bs, self.context_len = model, max_bs, context_len
@@ -62,6 +64,10 @@ class ModelRunner:
             torch.cuda.set_device(device_ids[0] if device_ids else 0)
         self.device = torch.device("cuda", torch.cuda.current_device())
         self._config_override = config
+        # `dtype`: the activations' format, overriding the checkpoint's ("bfloat16", "float16", or "float32" for the
+        # models that have float32 kernels throughout)
+        self._dtype_override = _DTYPES[dtype] if dtype else None
+        self.state_slots: Optional[int] = None      # set by load_model for models with per-sequence state
         self.graph: Optional[HIPGraph] = None
         self.block_table: Optional[BlockTable] = None
         self._sp_key, self._sp_dev, self._sp_unfiltered = None, None, False
@@ -81,21 +87,37 @@ class ModelRunner:
         # The kernels are built for bfloat16 and for float16 (the reference resolves the dtype from the checkpoint and
         # defaults to float16, model_runner.py:14-23,38-39); a float32 checkpoint is served in bfloat16 (same exponent
         # range), its tensors converted as they are loaded.
+        model_cls = model_class_of(cfg)
+        self.family = getattr(model_cls, "family", "paged_kv")
         self.checkpoint_dtype = _DTYPES[cfg.torch_dtype]
-        self.dtype = self.checkpoint_dtype if self.checkpoint_dtype in (torch.bfloat16, torch.float16) else torch.bfloat16
-        if self.checkpoint_dtype != self.dtype and self.rank == 0:
-            print(f"[nano_vllm_x_amd] checkpoint dtype {cfg.torch_dtype}: weights are converted to bfloat16", file=sys.stderr, flush=True)
-        self.num_heads, self.num_kv_heads, self.head_dim = get_model_config_per_gpu(cfg, self.tp_size)
+        wanted = self._dtype_override or self.checkpoint_dtype
+        if self.family == "seq_state":
+            # these models' kernels take the activations' format as an argument, float32 included (true float32: the
+            # library products of float32 tensors use no reduced-precision mode)
+            self.dtype = wanted
+            if self.dtype == torch.float32:
+                torch.backends.cuda.matmul.allow_tf32 = False
+                torch.set_float32_matmul_precision("highest")
+        else:
+            if self._dtype_override == torch.float32:
+                raise NotImplementedError("the paged-attention kernels are built for bfloat16 and float16 only")
+            self.dtype = wanted if wanted in (torch.bfloat16, torch.float16) else torch.bfloat16
+            if self.checkpoint_dtype != self.dtype and self._dtype_override is None and self.rank == 0:
+                print(f"[nano_vllm_x_amd] checkpoint dtype {cfg.torch_dtype}: weights are converted to bfloat16", file=sys.stderr, flush=True)
+            self.num_heads, self.num_kv_heads, self.head_dim = get_model_config_per_gpu(cfg, self.tp_size)
         prev = torch.get_default_dtype()
         torch.set_default_dtype(self.dtype)
         try:
             with torch.device(self.device):
-                self.model = Qwen3ForCausalLM(cfg)
+                self.model = model_cls(cfg)
         finally:
             torch.set_default_dtype(prev)
         self.model.finalize()
         self.model.eval()
-        self.start_layer, self.end_layer = self.model.model.start_layer, self.model.model.end_layer
+        stack = self.model.model if self.family == "paged_kv" else self.model
+        self.start_layer, self.end_layer = stack.start_layer, stack.end_layer
+        if self.family == "seq_state":
+            self.state_slots = self.max_bs
         self.num_layers = self.end_layer - self.start_layer     # of this pipeline stage
         if state_dict_iter is not None:
             self.model.load_weights(state_dict_iter)
@@ -111,7 +133,7 @@ class ModelRunner:
         # (ops.lmhead_sample): the tiled copy of this rank's LM-head rows it streams is made here, once.  NVX_LMHEAD_FUSED=0
         # keeps the two-launch path (library projection + sampler) everywhere.
         self._lmhead_packed = None
-        if (os.environ.get("NVX_LMHEAD_FUSED", "1") != "0" and tpd.pp_is_last() and cfg.hidden_size == 1024
+        if (self.family == "paged_kv" and os.environ.get("NVX_LMHEAD_FUSED", "1") != "0" and tpd.pp_is_last() and cfg.hidden_size == 1024
                 and self.dtype in (torch.bfloat16, torch.float16)):
             w = self.model.lm_head.weight
             self._lmhead_packed = ops.lmhead_pack(w.detach())
@@ -122,16 +144,37 @@ class ModelRunner:
         tpd.init_peer_allreduce(self.max_bs, cfg.hidden_size, self.dtype, self.device)
 
     def profile_kv_cache_size(self, gpu_memory_utilization: float = 0.9) -> int:
-        per_token = self.num_layers * self.num_kv_heads * self.head_dim * 2 * self.dtype.itemsize
+        if self.family == "seq_state":
+            from .kv_cache import LatentCachePool
+            # at least one byte per token: a model without a latent-attention layer caches nothing per token, and the pool's
+            # size then only bounds the slot numbers the scheduler hands out
+            per_token = max(LatentCachePool.bytes_per_token(self.model.latent_ranks(), self.dtype), 1)
+            cap = 1 << 24 if per_token == 1 else None
+        else:
+            per_token, cap = self.num_layers * self.num_kv_heads * self.head_dim * 2 * self.dtype.itemsize, None
         gc.collect()
         torch.cuda.empty_cache()
         free, _total = torch.cuda.mem_get_info(self.device)
         # ranks that share a device (rehearsals of several ranks on a one-GPU box) share its free memory too
         n = int(free * gpu_memory_utilization / tpd.ranks_on_my_device(self.device)) // per_token
+        if cap is not None:
+            n = min(n, cap)
         return tpd.tp_all_gather_min_int(n, self.device)
 
     def initialize_kv_cache(self, kv_cache_size: int):
         self.kv_cache_size = kv_cache_size
+        self._sample_out = torch.zeros(self.max_bs, dtype=torch.int64, device=self.device)
+        # two pinned landing buffers with an event each: a step queued behind another must not overwrite the
+        # ids the host has not read yet, and the host waits for ITS step's ids, not for the whole stream
+        self._sample_hosts = [torch.zeros(self.max_bs, dtype=torch.int64, pin_memory=True) for _ in range(2)]
+        self._sample_events = [torch.cuda.Event() for _ in range(2)]
+        self._sample_turn = 0
+        if self.family == "seq_state":
+            # a latent per token and latent-attention layer, one state slot per running sequence; steps run kernel by kernel
+            self.kv_cache = SeqStateCache(self.dtype, self.device, kv_cache_size, self.state_slots, self.model.latent_ranks(),
+                                          self.model.state_shapes())
+            self.attn_backend = SeqStateBackend(self.kv_cache, self.device)
+            return
         self.kv_cache = KVCachePool(dtype=self.dtype, device=self.device, num_tokens=kv_cache_size,
                                     num_layers=self.num_layers, num_heads=self.num_kv_heads, head_dim=self.head_dim,
                                     start_layer=self.start_layer, end_layer=self.end_layer)
@@ -141,12 +184,6 @@ class ModelRunner:
         n_rows = max(1024, 4 * self.max_bs) + 1
         self.block_table = BlockTable(self.max_bs, n_rows, 2 * self.context_len, self.device)
         self.decode_ws = ops.DecodeWorkspace(self.max_bs, self.num_heads, self.num_kv_heads, self.device)
-        self._sample_out = torch.zeros(self.max_bs, dtype=torch.int64, device=self.device)
-        # two pinned landing buffers with an event each: a step queued behind another must not overwrite the
-        # ids the host has not read yet, and the host waits for ITS step's ids, not for the whole stream
-        self._sample_hosts = [torch.zeros(self.max_bs, dtype=torch.int64, pin_memory=True) for _ in range(2)]
-        self._sample_events = [torch.cuda.Event() for _ in range(2)]
-        self._sample_turn = 0
         if not self.enforce_eager:
             self.graph = HIPGraph()
             try:
@@ -195,6 +232,8 @@ class ModelRunner:
 
     @staticmethod
     def prepare_last_hidden_states(batch: ForwardBatch, hidden_states: torch.Tensor) -> torch.Tensor:
+        if batch.want_rows is not None:     # the caller names the rows (any tokens of the step, in any number)
+            return hidden_states[torch.tensor(batch.want_rows, dtype=torch.int64).to(hidden_states.device)]
         last = np.cumsum([len(s.token_ids) - s.cached_kv_len for s in batch.seqs]) - 1
         if len(last) == hidden_states.shape[0]:
             return hidden_states   # decode: every row is a last row
@@ -204,7 +243,7 @@ class ModelRunner:
     @torch.inference_mode()
     def graph_step_possible(self, batch: ForwardBatch) -> bool:
         return batch.forward_mode == ForwardMode.DECODE and self.graph is not None and self.graph.is_captured \
-            and batch.num_seqs <= self.graph.max_bs and self.block_table.fits(batch.seqs)
+            and batch.want_rows is None and batch.num_seqs <= self.graph.max_bs and self.block_table.fits(batch.seqs)
 
     @torch.inference_mode()
     def compute_logits(self, batch: ForwardBatch, ids_on_device=None, shard: bool = False):
@@ -360,7 +399,7 @@ class ModelRunner:
         # keep the device block table in step with what the scheduler decided: rows are (re)written from the
         # step's own slot lists, sequence by sequence, so a decode step that had to run outside the graph
         # (no free row, a list longer than a row) does not keep its batch off the graph path afterwards
-        if self.graph is not None:
+        if self.graph is not None and self.family == "paged_kv":
             t = self.attn_backend.last_table
             self.block_table.write_rows(batch.seqs, t["paged_kv_indices"], t["paged_kv_indptr"])
         return hidden

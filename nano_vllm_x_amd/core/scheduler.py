@@ -36,12 +36,19 @@ from collections import deque
 from typing import Callable, Deque, Optional
 
 from .common import ForwardBatch, ForwardMode, Sequence, SequenceStatus
-from .kv_cache import KVCacheManager
+from .kv_cache import KVCacheManager, StateSlotAllocator
 
 
 class Scheduler:
     def __init__(self, kv_cache_size: int, max_bs: int = 32, prefix_reuse: bool = False,
-                 max_prefill_tokens: Optional[int] = None, chunked_prefill: bool = False):
+                 max_prefill_tokens: Optional[int] = None, chunked_prefill: bool = False, state_slots: Optional[int] = None):
+        # `state_slots`: the model keeps per-sequence state besides its per-token cache rows (a recurrence, the tail of a
+        # convolution), in that many slots.  A sequence then holds a state slot from admission until it finishes or is
+        # preempted, admission waits for a free one, and cached rows are not kept for later requests: a prefix's rows are
+        # of no use without the state at its end, so a finished sequence's slots go straight back to the allocator.
+        if state_slots is not None and prefix_reuse:
+            raise ValueError("prefix_reuse cannot serve a model with per-sequence state: the state at the end of a cached prefix is not kept")
+        self.state_slots = StateSlotAllocator(state_slots) if state_slots is not None else None
         self.kv_cache_size = kv_cache_size
         self.max_bs = max_bs
         self.prefix_reuse = prefix_reuse
@@ -88,6 +95,17 @@ class Scheduler:
             seq.kv_indices.clear()
             seq.cached_kv_len = 0
 
+    def _take_state_slot(self, seq: Sequence) -> bool:
+        if self.state_slots is None:
+            return True
+        seq.state_slot = self.state_slots.alloc(seq.seq_id)
+        return seq.state_slot is not None
+
+    def _drop_state_slot(self, seq: Sequence):
+        if self.state_slots is not None:
+            self.state_slots.free(seq.seq_id)
+            seq.state_slot = None
+
     # -- one step ---------------------------------------------------------------------------------
     def schedule(self) -> Optional[ForwardBatch]:
         if self.chunked_prefill:
@@ -118,6 +136,11 @@ class Scheduler:
                 if sum(len(s.token_ids) - s.cached_kv_len for s in picked) + len(head.token_ids) > budget:
                     break
             seq = self.waiting.popleft()
+            if not self._take_state_slot(seq):
+                self.waiting.appendleft(seq)
+                if not picked and not self.running:
+                    raise RuntimeError("no state slot is free and nothing is running that could release one")
+                break
             try:
                 if self.prefix_reuse and not seq.kv_indices:
                     self.kv_manager.adopt_cached_prefix(seq)
@@ -125,6 +148,7 @@ class Scheduler:
             except RuntimeError:
                 if self.prefix_reuse:
                     self.kv_manager.release_sequence(seq)
+                self._drop_state_slot(seq)
                 self.waiting.appendleft(seq)
                 if not picked and not self.running:
                     raise
@@ -143,6 +167,7 @@ class Scheduler:
                         token_ids=seq.token_ids[:end], sampling_params=seq.sampling_params, kv_indices=seq.kv_indices[:end],
                         cached_kv_len=seq.cached_kv_len)
         view.partial_of = seq
+        view.state_slot = seq.state_slot
         return view
 
     def _schedule_chunks(self):
@@ -162,6 +187,11 @@ class Scheduler:
             picked.append(seq if take == left else self._chunk_view(seq, seq.cached_kv_len + take))
         while self.waiting and len(picked) < self.max_bs and budget > 0:
             seq = self.waiting.popleft()
+            if not self._take_state_slot(seq):
+                self.waiting.appendleft(seq)
+                if not picked and not self.running:
+                    raise RuntimeError("no state slot is free and nothing is running that could release one")
+                break
             try:
                 if self.prefix_reuse and not seq.kv_indices:
                     self.kv_manager.adopt_cached_prefix(seq)
@@ -169,6 +199,7 @@ class Scheduler:
             except RuntimeError:
                 if self.prefix_reuse:
                     self.kv_manager.release_sequence(seq)
+                self._drop_state_slot(seq)
                 self.waiting.appendleft(seq)
                 if not picked and not self.running:
                     raise
@@ -185,6 +216,48 @@ class Scheduler:
                 self.prefilling[seq.seq_id] = seq
                 picked.append(self._chunk_view(seq, seq.cached_kv_len + take))
         return picked
+
+    # -- a step given from outside --------------------------------------------------------------------
+    def schedule_given(self, plan) -> Optional[ForwardBatch]:
+        """One step whose content is given instead of chosen: `plan` lists (seq_id, n) pairs, the next n tokens of each
+        of these sequences (a replayed trace, a front end with a policy of its own).  The mechanisms are the scheduler's
+        own: a waiting sequence is admitted (state slot, token slots for all its tokens), a sequence whose tokens go
+        beyond the n asked for is shown to the model as a chunk view.  Portions of prompts and single tokens of running
+        sequences share the batch; it is a DECODE batch if every entry continues its sequence by one token.
+        commit_given() completes the step."""
+        picked = []
+        for seq_id, n in plan:
+            seq = self.sequences[seq_id]
+            if seq_id in self.scheduled:
+                raise RuntimeError(f"sequence {seq_id!r} is already part of a step in flight")
+            if n < 1 or seq.cached_kv_len + n > len(seq.token_ids):
+                raise ValueError(f"sequence {seq_id!r}: {n} tokens asked for, {len(seq.token_ids) - seq.cached_kv_len} are waiting")
+            if seq.status == SequenceStatus.WAITING:
+                if not self._take_state_slot(seq):
+                    raise RuntimeError("no state slot is free")
+                self.waiting.remove(seq)
+                seq.status = SequenceStatus.RUNNING
+                self.running.append(seq)
+            try:
+                self.alloc_kv_slots(seq)
+            except RuntimeError:
+                for s in picked:
+                    self.scheduled.discard(s.seq_id)
+                raise
+            self.scheduled.add(seq_id)
+            end = seq.cached_kv_len + n
+            picked.append(seq if end == len(seq.token_ids) else self._chunk_view(seq, end))
+        if not picked:
+            return None
+        decode = all(s.partial_of is None and s.cached_kv_len > 0 and len(s.token_ids) - s.cached_kv_len == 1 for s in picked)
+        return ForwardBatch(forward_mode=ForwardMode.DECODE if decode else ForwardMode.PREFILL, num_seqs=len(picked), seqs=picked)
+
+    def commit_given(self, batch: ForwardBatch):
+        """The step of schedule_given has run: its tokens have their rows; no token is appended."""
+        for s in batch.seqs:
+            seq = s.partial_of if s.partial_of is not None else s
+            self.scheduled.discard(seq.seq_id)
+            seq.cached_kv_len = len(s.token_ids)
 
     def finish_chunk(self, view: Sequence):
         """A chunk step has run: the rows up to the view's end are written; the sampled token is dropped."""
@@ -243,6 +316,7 @@ class Scheduler:
         self.scheduled.discard(seq.seq_id)
         self.prefilling.pop(seq.seq_id, None)
         self.free_kv_slots(seq)
+        self._drop_state_slot(seq)     # the recomputation starts from position 0, where no state is read
         seq.status = SequenceStatus.WAITING
         self.waiting.appendleft(seq)
         if self.on_release:
@@ -286,9 +360,11 @@ class Scheduler:
             self.running.remove(seq)
             self.scheduled.discard(seq.seq_id)
         seq.status = SequenceStatus.FINISHED
-        if self.prefilling.pop(seq.seq_id, None) is not None:
+        self._drop_state_slot(seq)
+        if self.prefilling.pop(seq.seq_id, None) is not None or self.state_slots is not None:
             # aborted with its prompt only partly computed: the rows past cached_kv_len hold nothing, so the
-            # sequence gives its slots back instead of entering the prefix tree
+            # sequence gives its slots back instead of entering the prefix tree (as does every sequence of a model with
+            # per-sequence state)
             if self.prefix_reuse:
                 self.kv_manager.release_sequence(seq)
             else:

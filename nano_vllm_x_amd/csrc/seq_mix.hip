@@ -1,0 +1,321 @@
+// Kernels of layer stacks that keep a 32-bit residual stream and per-sequence recurrent state:
+//   - boundary norm: post-norm of a sublayer's output + residual add (+ weighted sum over the results of all layers so
+//     far) + pre-norm of the next sublayer, one launch per sublayer boundary;
+//   - short causal convolution over time on every channel ("canon"), its tail of inputs kept per sequence;
+//   - gated linear recurrence with state-independent gates (minGRU);
+//   - squared ReLU.
+// Activations (`fmt`: 0 bfloat16, 1 float16, 2 float32) are what the matrix products read and write; norm weights,
+// convolution taps, mixing weights, the residual stream and every state are float32 in all formats.
+// A batch is a ragged list of sequences: tokens [qo_indptr[b], qo_indptr[b+1]) belong to sequence b, whose first token
+// of this step stands at position pos0[b] and whose state lives in slot state_slot[b] (a negative slot: a padding row,
+// nothing is read or written).  A sequence at position 0 has no state yet: the kernels take zeros instead of reading it,
+// so a slot needs no clearing when it is handed to a new sequence.
+#include "nvx_dev.h"
+
+namespace NVX_NS {
+
+template <typename A> __device__ __forceinline__ float ldf(const A* p, int64_t i) { return (float)p[i]; }
+template <typename A> __device__ __forceinline__ void stf(A* p, int64_t i, float v) { p[i] = (A)v; }
+
+// sum over a workgroup of 256 threads; every thread gets the total.  `red` holds 4 floats; safe to call repeatedly.
+__device__ __forceinline__ float block_sum256(float v, float* red) {
+    v = wave_sum(v);
+    __syncthreads();                       // the previous call's readers are done
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return red[0] + red[1] + red[2] + red[3];
+}
+
+// ---- boundary norm ------------------------------------------------------------------------------------------------
+// Per token t (one workgroup each):
+//   r   = res[t] + m[t] / rms(m[t]) * (1 + w_post)                 (res == null: r = the normed m alone)
+//   hist[hist_slot][t] = r                                          (hist_slot >= 0)
+//   x   = sum_{j < n_mix} mix[j] * hist[j][t]                       (n_mix > 0; hist[hist_slot] is r), else x = r
+//   x_out[t] = x
+//   y   = x / rms(x) * (1 + w_pre)  ->  y_f32[t] (float) or y_act[t] (activation format), whichever is given
+template <typename A>
+__global__ __launch_bounds__(256) void boundary_norm_kernel(
+    const A* __restrict__ m, int64_t m_stride, const float* __restrict__ res, const float* __restrict__ w_post,
+    float* __restrict__ hist, int64_t hist_stride, int hist_slot, int n_mix, const float* __restrict__ mix,
+    float* __restrict__ x_out, const float* __restrict__ w_pre, float* __restrict__ y_f32, A* __restrict__ y_act,
+    int width, float eps) {
+    __shared__ float red[4];
+    const int64_t t = blockIdx.x;
+    const A* mr = m + t * m_stride;
+    const int64_t row = t * (int64_t)width;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < width; c += 256) { const float v = ldf(mr, c); ss += v * v; }
+    const float r_post = 1.0f / sqrtf(block_sum256(ss, red) / (float)width + eps);
+    float ss2 = 0.f;
+    for (int c = threadIdx.x; c < width; c += 256) {
+        float r = ldf(mr, c) * r_post * (1.0f + w_post[c]);
+        if (res) r += res[row + c];
+        if (hist_slot >= 0) hist[(int64_t)hist_slot * hist_stride + row + c] = r;
+        float x = r;
+        if (n_mix > 0) {
+            x = 0.f;
+            for (int j = 0; j < n_mix; ++j)
+                x += mix[j] * (j == hist_slot ? r : hist[(int64_t)j * hist_stride + row + c]);
+        }
+        x_out[row + c] = x;
+        ss2 += x * x;
+    }
+    if (!w_pre) return;
+    const float r_pre = 1.0f / sqrtf(block_sum256(ss2, red) / (float)width + eps);
+    for (int c = threadIdx.x; c < width; c += 256) {
+        const float y = x_out[row + c] * r_pre * (1.0f + w_pre[c]);   // this thread's own store, read back
+        if (y_f32) y_f32[row + c] = y;
+        else stf(y_act, row + c, y);
+    }
+}
+
+// ---- canon: h + causal convolution over time, per channel -----------------------------------------------------------
+// taps[c][j] multiplies the input (taps_n - 1 - j) tokens back.  state[slot][r] (r < taps_n - 1) is the input at position
+// pos0 - (taps_n - 1) + r.
+template <typename A>
+__global__ __launch_bounds__(256) void canon_conv_kernel(
+    const float* __restrict__ h, const float* __restrict__ taps, int taps_n, const float* __restrict__ state,
+    const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ qo_indptr, const int64_t* __restrict__ pos0,
+    const int32_t* __restrict__ state_slot, A* __restrict__ out, int64_t n_tok, int width) {
+    const int64_t total = n_tok * (int64_t)width;
+    for (int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x; id < total; id += (int64_t)gridDim.x * 256) {
+        const int64_t t = id / width;
+        const int c = (int)(id - t * width);
+        const int b = tok_seq ? tok_seq[t] : (int)t;
+        const int slot = state_slot[b];
+        if (slot < 0) { stf(out, id, 0.f); continue; }
+        const int64_t q0 = qo_indptr ? qo_indptr[b] : t;
+        const int64_t local = t - q0;
+        const bool has_state = pos0[b] > 0;
+        const int hist_n = taps_n - 1;
+        float acc = h[id];
+        for (int j = 0; j < taps_n; ++j) {
+            const int64_t s = local - hist_n + j;
+            float v;
+            if (s >= 0) v = h[(q0 + s) * width + c];
+            else v = has_state ? state[((int64_t)slot * hist_n + (hist_n + s)) * width + c] : 0.f;
+            acc += taps[(int64_t)c * taps_n + j] * v;
+        }
+        stf(out, id, acc);
+    }
+}
+
+// After the convolution has read the old tail: the last taps_n - 1 inputs of every sequence become its new tail.
+__global__ __launch_bounds__(256) void canon_state_kernel(
+    const float* __restrict__ h, int taps_n, float* __restrict__ state, const int32_t* __restrict__ qo_indptr,
+    const int64_t* __restrict__ pos0, const int32_t* __restrict__ state_slot, int width) {
+    const int b = blockIdx.y;
+    const int slot = state_slot[b];
+    if (slot < 0) return;
+    const int64_t q0 = qo_indptr ? qo_indptr[b] : b;
+    const int64_t n = qo_indptr ? qo_indptr[b + 1] - q0 : 1;
+    if (n <= 0) return;
+    const bool has_state = pos0[b] > 0;
+    const int hist_n = taps_n - 1;
+    for (int c = blockIdx.x * 256 + threadIdx.x; c < width; c += gridDim.x * 256) {
+        float* st = state + (int64_t)slot * hist_n * width + c;
+        for (int r = 0; r < hist_n; ++r) {        // ascending: row r takes old row r + n, which is not yet overwritten
+            const int64_t s = n - hist_n + r;
+            float v;
+            if (s >= 0) v = h[(q0 + s) * width + c];
+            else v = has_state ? st[(int64_t)(r + n) * width] : 0.f;
+            st[(int64_t)r * width] = v;
+        }
+    }
+}
+
+// ---- squared ReLU ---------------------------------------------------------------------------------------------------
+template <typename A>
+__global__ __launch_bounds__(256) void relu2_kernel(const A* __restrict__ x, A* __restrict__ y, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+        const float v = fmaxf(ldf(x, i), 0.f);
+        stf(y, i, v * v);
+    }
+}
+
+// ---- minGRU ---------------------------------------------------------------------------------------------------------
+// zxg[t] = [ z pre-activation | candidate pre-activation u | output-gate pre-activation g ], `width` each.
+//   z = sigmoid(.),  cand = u + 1/2 (u >= 0) or sigmoid(u) (u < 0),  S <- (1 - z) S + z cand,  out = S * silu(g)
+// The recurrence is S_t = a_t S_(t-1) + b_t with a = 1 - z, b = z cand.  A workgroup takes 64 channels of one sequence
+// and walks its tokens in rounds of SEG * 4 tokens: each of its 4 waves scans SEG consecutive tokens from a zero
+// state (keeping the running product of a), the four partial results are chained through LDS, and every wave then adds
+// its incoming state times the running product.  All of it in float32.
+__device__ __forceinline__ float sigmoidf_(float v) { return 1.0f / (1.0f + expf(-v)); }
+
+template <typename A, int SEG>
+__global__ __launch_bounds__(256) void mingru_scan_kernel(
+    const A* __restrict__ zxg, int64_t row_stride, float* __restrict__ state, const int32_t* __restrict__ qo_indptr,
+    const int64_t* __restrict__ pos0, const int32_t* __restrict__ state_slot, A* __restrict__ out, int width) {
+    __shared__ float agg_a[4][64], agg_b[4][64];
+    const int b = blockIdx.y;
+    const int slot = state_slot[b];
+    if (slot < 0) return;
+    const int64_t q0 = qo_indptr ? qo_indptr[b] : b;
+    const int64_t n = qo_indptr ? qo_indptr[b + 1] - q0 : 1;
+    if (n <= 0) return;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int c = blockIdx.x * 64 + lane;
+    const bool live = c < width;
+    float carry = (live && pos0[b] > 0) ? state[(int64_t)slot * width + c] : 0.f;
+    for (int64_t base = 0; base < n; base += SEG * 4) {
+        const int64_t t0 = base + (int64_t)wv * SEG;
+        float pa[SEG], ps[SEG], gg[SEG];
+        float a_run = 1.f, s_run = 0.f;
+#pragma unroll
+        for (int i = 0; i < SEG; ++i) {
+            const int64_t t = t0 + i;
+            if (live && t < n) {
+                const A* r = zxg + (q0 + t) * row_stride;
+                const float z = sigmoidf_(ldf(r, c));
+                const float u = ldf(r, (int64_t)width + c);
+                const float cand = u >= 0.f ? u + 0.5f : sigmoidf_(u);
+                const float g = ldf(r, 2 * (int64_t)width + c);
+                gg[i] = g * sigmoidf_(g);
+                s_run = (1.0f - z) * s_run + z * cand;
+                a_run *= (1.0f - z);
+            } else gg[i] = 0.f;
+            pa[i] = a_run;
+            ps[i] = s_run;
+        }
+        __syncthreads();                   // the previous round's readers are done
+        agg_a[wv][lane] = a_run;
+        agg_b[wv][lane] = s_run;
+        __syncthreads();
+        float in = carry;                  // state before this wave's first token
+        for (int k = 0; k < wv; ++k) in = agg_a[k][lane] * in + agg_b[k][lane];
+        float last = in;
+        for (int k = wv; k < 4; ++k) last = agg_a[k][lane] * last + agg_b[k][lane];
+        carry = last;                      // state after the round's last token (segments past the end are identities)
+#pragma unroll
+        for (int i = 0; i < SEG; ++i) {
+            const int64_t t = t0 + i;
+            if (live && t < n) stf(out, (q0 + t) * (int64_t)width + c, (pa[i] * in + ps[i]) * gg[i]);
+        }
+    }
+    if (live && wv == 0) state[(int64_t)slot * width + c] = carry;
+}
+
+// one token per sequence (a decode step): thread = (sequence, channel)
+template <typename A>
+__global__ __launch_bounds__(256) void mingru_step_kernel(
+    const A* __restrict__ zxg, int64_t row_stride, float* __restrict__ state, const int64_t* __restrict__ pos0,
+    const int32_t* __restrict__ state_slot, A* __restrict__ out, int64_t n_seq, int width) {
+    const int64_t total = n_seq * (int64_t)width;
+    for (int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x; id < total; id += (int64_t)gridDim.x * 256) {
+        const int64_t b = id / width;
+        const int c = (int)(id - b * width);
+        const int slot = state_slot[b];
+        if (slot < 0) { stf(out, id, 0.f); continue; }
+        const A* r = zxg + b * row_stride;
+        const float z = sigmoidf_(ldf(r, c));
+        const float u = ldf(r, (int64_t)width + c);
+        const float cand = u >= 0.f ? u + 0.5f : sigmoidf_(u);
+        const float g = ldf(r, 2 * (int64_t)width + c);
+        float* sp = state + (int64_t)slot * width + c;
+        const float s = (1.0f - z) * (pos0[b] > 0 ? *sp : 0.f) + z * cand;
+        *sp = s;
+        stf(out, id, s * (g * sigmoidf_(g)));
+    }
+}
+
+template <typename A>
+static void launch_boundary(const void* m, int64_t m_stride, const float* res, const float* w_post, float* hist, int64_t hist_stride,
+                            int hist_slot, int n_mix, const float* mix, float* x_out, const float* w_pre, float* y_f32, void* y_act,
+                            int64_t n_tok, int width, float eps, hipStream_t s) {
+    hipLaunchKernelGGL(boundary_norm_kernel<A>, dim3((unsigned)n_tok), dim3(256), 0, s, (const A*)m, m_stride, res, w_post, hist,
+                       hist_stride, hist_slot, n_mix, mix, x_out, w_pre, y_f32, (A*)y_act, width, eps);
+}
+
+template <typename A>
+static void launch_canon(const float* h, const float* taps, int taps_n, float* state, const int32_t* tok_seq, const int32_t* qo_indptr,
+                         const int64_t* pos0, const int32_t* state_slot, void* out, int64_t n_tok, int64_t n_seq, int width,
+                         hipStream_t s) {
+    int64_t blocks = (n_tok * width + 255) / 256;
+    if (blocks > 256 * 64) blocks = 256 * 64;
+    hipLaunchKernelGGL(canon_conv_kernel<A>, dim3((unsigned)blocks), dim3(256), 0, s, h, taps, taps_n, (const float*)state, tok_seq,
+                       qo_indptr, pos0, state_slot, (A*)out, n_tok, width);
+    if (taps_n > 1)
+        hipLaunchKernelGGL(canon_state_kernel, dim3((unsigned)((width + 255) / 256), (unsigned)n_seq), dim3(256), 0, s, h, taps_n, state,
+                           qo_indptr, pos0, state_slot, width);
+}
+
+template <typename A>
+static void launch_mingru(const void* zxg, int64_t row_stride, float* state, const int32_t* qo_indptr, const int64_t* pos0,
+                          const int32_t* state_slot, void* out, int64_t n_seq, int width, hipStream_t s) {
+    if (!qo_indptr) {
+        int64_t blocks = (n_seq * width + 255) / 256;
+        if (blocks > 256 * 64) blocks = 256 * 64;
+        hipLaunchKernelGGL(mingru_step_kernel<A>, dim3((unsigned)blocks), dim3(256), 0, s, (const A*)zxg, row_stride, state, pos0,
+                           state_slot, (A*)out, n_seq, width);
+        return;
+    }
+    hipLaunchKernelGGL((mingru_scan_kernel<A, 8>), dim3((unsigned)((width + 63) / 64), (unsigned)n_seq), dim3(256), 0, s, (const A*)zxg,
+                       row_stride, state, qo_indptr, pos0, state_slot, (A*)out, width);
+}
+
+}  // namespace NVX_NS
+
+using namespace NVX_NS;
+
+#define NVX_FMT_DISPATCH(fmt, CALL)                                         \
+    do {                                                                    \
+        if ((fmt) == 0) { typedef __bf16 A_; CALL; }                        \
+        else if ((fmt) == 1) { typedef _Float16 A_; CALL; }                 \
+        else { typedef float A_; CALL; }                                    \
+    } while (0)
+
+extern "C" int nvx_boundary_norm(const void* m, int64_t m_row_stride, int fmt, const float* res, const float* w_post, float* hist,
+                                 int64_t hist_stride, int hist_slot, int n_mix, const float* mix, float* x_out, const float* w_pre,
+                                 float* y_f32, void* y_act, int64_t n_tok, int64_t width, float eps, nvx_stream_t stream) {
+    NVX_REQUIRE(fmt >= 0 && fmt <= 2, NVX_EINVAL, "nvx_boundary_norm: fmt must be 0 (bfloat16), 1 (float16) or 2 (float32)");
+    NVX_REQUIRE(n_tok >= 0 && width > 0 && width < (1 << 30) && m_row_stride >= width, NVX_EINVAL, "nvx_boundary_norm: bad sizes");
+    if (n_tok == 0) return NVX_OK;
+    NVX_REQUIRE(m && w_post && x_out, NVX_EINVAL, "nvx_boundary_norm: null pointer");
+    NVX_REQUIRE(hist_slot < 0 || hist, NVX_EINVAL, "nvx_boundary_norm: hist_slot without a history buffer");
+    NVX_REQUIRE(n_mix == 0 || (hist && mix && hist_slot >= 0 && hist_slot < n_mix), NVX_EINVAL,
+                "nvx_boundary_norm: mixing needs the history buffer, the weights and this result's slot among them");
+    NVX_REQUIRE(!hist || hist_stride >= n_tok * width, NVX_EINVAL, "nvx_boundary_norm: history stride smaller than a result");
+    NVX_REQUIRE(!w_pre || (y_f32 != nullptr) != (y_act != nullptr), NVX_EINVAL, "nvx_boundary_norm: exactly one output for the pre-norm");
+    NVX_FMT_DISPATCH(fmt, launch_boundary<A_>(m, m_row_stride, res, w_post, hist, hist_stride, hist_slot, n_mix, mix, x_out, w_pre, y_f32,
+                                              y_act, n_tok, (int)width, eps, (hipStream_t)stream));
+    return nvx_check_launch("nvx_boundary_norm");
+}
+
+extern "C" int nvx_canon_conv(const float* h, const float* taps, int taps_n, float* state, int64_t n_slots, const int32_t* tok_seq,
+                              const int32_t* qo_indptr, const int64_t* pos0, const int32_t* state_slot, void* out, int fmt,
+                              int64_t n_tok, int64_t n_seq, int64_t width, nvx_stream_t stream) {
+    NVX_REQUIRE(fmt >= 0 && fmt <= 2, NVX_EINVAL, "nvx_canon_conv: fmt must be 0, 1 or 2");
+    NVX_REQUIRE(n_tok >= 0 && n_seq >= 0 && n_seq <= 65535 && width > 0 && width < (1 << 30) && taps_n >= 1 && taps_n <= 64 && n_slots >= 0,
+                NVX_EINVAL, "nvx_canon_conv: bad sizes");
+    if (n_tok == 0 || n_seq == 0) return NVX_OK;
+    NVX_REQUIRE(h && taps && out && pos0 && state_slot && (state || taps_n == 1), NVX_EINVAL, "nvx_canon_conv: null pointer");
+    NVX_REQUIRE((tok_seq != nullptr) == (qo_indptr != nullptr), NVX_EINVAL, "nvx_canon_conv: tok_seq and qo_indptr go together");
+    NVX_REQUIRE(qo_indptr || n_tok == n_seq, NVX_EINVAL, "nvx_canon_conv: without qo_indptr every sequence has one token");
+    NVX_FMT_DISPATCH(fmt, launch_canon<A_>(h, taps, taps_n, state, tok_seq, qo_indptr, pos0, state_slot, out, n_tok, n_seq, (int)width,
+                                           (hipStream_t)stream));
+    return nvx_check_launch("nvx_canon_conv");
+}
+
+extern "C" int nvx_relu2(const void* x, void* y, int fmt, int64_t n, nvx_stream_t stream) {
+    NVX_REQUIRE(fmt >= 0 && fmt <= 2 && n >= 0, NVX_EINVAL, "nvx_relu2: bad arguments");
+    if (n == 0) return NVX_OK;
+    NVX_REQUIRE(x && y, NVX_EINVAL, "nvx_relu2: null pointer");
+    int64_t blocks = (n + 255) / 256;
+    if (blocks > 256 * 64) blocks = 256 * 64;
+    NVX_FMT_DISPATCH(fmt, hipLaunchKernelGGL(relu2_kernel<A_>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const A_*)x,
+                                             (A_*)y, n));
+    return nvx_check_launch("nvx_relu2");
+}
+
+extern "C" int nvx_mingru_scan(const void* zxg, int64_t row_stride, int fmt, float* state, int64_t n_slots, const int32_t* qo_indptr,
+                               const int64_t* pos0, const int32_t* state_slot, void* out, int64_t n_tok, int64_t n_seq, int64_t width,
+                               nvx_stream_t stream) {
+    NVX_REQUIRE(fmt >= 0 && fmt <= 2, NVX_EINVAL, "nvx_mingru_scan: fmt must be 0, 1 or 2");
+    NVX_REQUIRE(n_tok >= 0 && n_seq >= 0 && n_seq <= 65535 && width > 0 && width < (1 << 30) && row_stride >= 3 * width && n_slots >= 0,
+                NVX_EINVAL, "nvx_mingru_scan: bad sizes");
+    if (n_tok == 0 || n_seq == 0) return NVX_OK;
+    NVX_REQUIRE(zxg && state && pos0 && state_slot && out, NVX_EINVAL, "nvx_mingru_scan: null pointer");
+    NVX_REQUIRE(qo_indptr || n_tok == n_seq, NVX_EINVAL, "nvx_mingru_scan: without qo_indptr every sequence has one token");
+    NVX_FMT_DISPATCH(fmt, launch_mingru<A_>(zxg, row_stride, state, qo_indptr, pos0, state_slot, out, n_seq, (int)width, (hipStream_t)stream));
+    return nvx_check_launch("nvx_mingru_scan");
+}

@@ -362,7 +362,7 @@ class AttentionBackend:
 @contextmanager
 def attention_kv_cache(model: nn.Module, metadata: AttentionMetadata):
     """Hand `metadata` to every Attention module of `model` for the duration of one forward."""
-    touched = [m for m in model.modules() if isinstance(m, Attention)]
+    touched = [m for m in model.modules() if hasattr(m, "set_attention_metadata")]
     for m in touched:
         m.set_attention_metadata(metadata)
     try:

@@ -665,3 +665,173 @@ def peer_allreduce_norm(group: PeerGroup, x, weight=None, eps: float = 0.0, resi
     _lib.check(_fn(lib, "nvx_peer_allreduce_norm", x.dtype)(group.comm, _ptr(x), x.stride(0), _ptr(residual), _ptr(weight), _ptr(y), _ptr(res_out),
                                                              rows, hidden, float(eps), _stream()), "nvx_peer_allreduce_norm")
     return y if residual is None else (y, res_out)
+
+
+# ---------------------------------------------------------------------------------------------
+# layers with a float32 residual stream, per-sequence state and latent attention
+# ---------------------------------------------------------------------------------------------
+F32 = torch.float32
+_FMT = {BF16: 0, F16: 1, F32: 2}
+
+
+def _fmt(t) -> int:
+    _need(t.dtype in _FMT, "activations must be bfloat16, float16 or float32")
+    return _FMT[t.dtype]
+
+
+def _f32c(t, what: str):
+    _need(t.dtype == F32 and t.is_contiguous(), f"{what} must be contiguous float32")
+
+
+class StepLayout:
+    """Where the tokens of a step belong: `qo_indptr` (int32, B+1) and `tok_seq` (int32, T) give each token its sequence
+    (both None: one token per sequence, a decode step), `pos0` (int64, B) the position of each sequence's first token of
+    the step, `state_slot` (int32, B) its slot in the state tensors (negative: a padding row)."""
+
+    def __init__(self, n_tok: int, n_seq: int, pos0, state_slot, qo_indptr=None, tok_seq=None):
+        _dev(pos0, state_slot, qo_indptr, tok_seq)
+        _need(pos0.dtype == torch.int64 and pos0.is_contiguous() and pos0.numel() >= n_seq, "StepLayout: pos0 must be int64 (B)")
+        _need(state_slot.dtype == torch.int32 and state_slot.is_contiguous() and state_slot.numel() >= n_seq,
+              "StepLayout: state_slot must be int32 (B)")
+        _need((qo_indptr is None) == (tok_seq is None), "StepLayout: qo_indptr and tok_seq go together")
+        if qo_indptr is None:
+            _need(n_tok == n_seq, "StepLayout: without qo_indptr every sequence has one token")
+        else:
+            _need(qo_indptr.dtype == torch.int32 and qo_indptr.is_contiguous() and qo_indptr.numel() == n_seq + 1, "StepLayout: qo_indptr")
+            _need(tok_seq.dtype == torch.int32 and tok_seq.is_contiguous() and tok_seq.numel() == n_tok, "StepLayout: tok_seq")
+        self.n_tok, self.n_seq = n_tok, n_seq
+        self.pos0, self.state_slot, self.qo_indptr, self.tok_seq = pos0, state_slot, qo_indptr, tok_seq
+
+
+def boundary_norm(m, w_post, eps: float, res=None, hist=None, hist_slot: int = -1, mix=None, w_pre=None, pre_f32: bool = True,
+                  x_out=None):
+    """Post-norm of a sublayer's output `m` (T, width) + residual `res` (float32) [+ weighted sum `mix` over the results
+    kept in `hist` (slots, T, width), this one stored at `hist_slot`] [+ pre-norm `w_pre` of what follows].  Both norms
+    are RMS norms whose stored weight is the deviation from one.  Returns (x, y): the new stream (float32) and the
+    pre-normed rows (float32 if `pre_f32`, else in m's format; None without `w_pre`)."""
+    _dev(m, w_post, res, hist, mix, w_pre)
+    _need(m.dim() == 2 and m.stride(1) == 1, "boundary_norm: m must be (T, width) with unit inner stride")
+    t, width = m.shape
+    _f32c(w_post, "boundary_norm: w_post")
+    _need(w_post.numel() == width, "boundary_norm: w_post size")
+    if res is not None:
+        _f32c(res, "boundary_norm: res")
+        _need(res.shape == (t, width), "boundary_norm: res shape")
+    n_mix, hist_stride = 0, 0
+    if hist is not None:
+        _f32c(hist, "boundary_norm: hist")
+        _need(hist.dim() == 3 and hist.shape[1:] == (t, width) and 0 <= hist_slot < hist.shape[0], "boundary_norm: hist shape / slot")
+        hist_stride = hist.stride(0)
+        if mix is not None:
+            _f32c(mix, "boundary_norm: mix")
+            n_mix = mix.numel()
+            _need(hist_slot < n_mix <= hist.shape[0], "boundary_norm: mix longer than the history, or without this result")
+    else:
+        _need(mix is None and hist_slot < 0, "boundary_norm: mix / hist_slot need hist")
+    if x_out is None:
+        x_out = torch.empty((t, width), dtype=F32, device=m.device)
+    else:
+        _f32c(x_out, "boundary_norm: x_out")
+        _need(x_out.shape == (t, width), "boundary_norm: x_out shape")
+    y = None
+    if w_pre is not None:
+        _f32c(w_pre, "boundary_norm: w_pre")
+        _need(w_pre.numel() == width, "boundary_norm: w_pre size")
+        y = torch.empty((t, width), dtype=F32 if pre_f32 else m.dtype, device=m.device)
+    lib = _lib.load()
+    _lib.check(lib.nvx_boundary_norm(_ptr(m), m.stride(0), _fmt(m), _ptr(res), _ptr(w_post), _ptr(hist), hist_stride, hist_slot, n_mix,
+                                     _ptr(mix), _ptr(x_out), _ptr(w_pre), _ptr(y) if (y is not None and pre_f32) else None,
+                                     _ptr(y) if (y is not None and not pre_f32) else None, t, width, float(eps), _stream()),
+               "nvx_boundary_norm")
+    return x_out, y
+
+
+def canon_conv(h, taps, state, layout: StepLayout, dtype):
+    """h + causal convolution over time per channel.  h (T, width) float32; taps (width, taps_n) float32; state
+    (slots, taps_n - 1, width) float32, read for the inputs before this step and replaced by each sequence's last ones.
+    Returns (T, width) in `dtype`."""
+    _dev(h, taps, state)
+    _f32c(h, "canon_conv: h")
+    _f32c(taps, "canon_conv: taps")
+    t, width = h.shape
+    taps_n = taps.shape[1]
+    _need(t == layout.n_tok and taps.shape[0] == width, "canon_conv: shapes")
+    n_slots = 0
+    if taps_n > 1:
+        _f32c(state, "canon_conv: state")
+        _need(state.dim() == 3 and state.shape[1:] == (taps_n - 1, width), "canon_conv: state shape")
+        n_slots = state.shape[0]
+    out = torch.empty((t, width), dtype=dtype, device=h.device)
+    lib = _lib.load()
+    _lib.check(lib.nvx_canon_conv(_ptr(h), _ptr(taps), taps_n, _ptr(state) if taps_n > 1 else None, n_slots, _ptr(layout.tok_seq),
+                                  _ptr(layout.qo_indptr), _ptr(layout.pos0), _ptr(layout.state_slot), _ptr(out), _fmt(out), t,
+                                  layout.n_seq, width, _stream()), "nvx_canon_conv")
+    return out
+
+
+def relu2(x):
+    """max(x, 0)^2."""
+    _dev(x)
+    x = x.contiguous()
+    y = torch.empty_like(x)
+    lib = _lib.load()
+    _lib.check(lib.nvx_relu2(_ptr(x), _ptr(y), _fmt(x), x.numel(), _stream()), "nvx_relu2")
+    return y
+
+
+def mingru_scan(zxg, state, layout: StepLayout):
+    """Gated recurrence over each sequence's tokens.  zxg (T, 3 * width): update-gate, candidate and output-gate
+    pre-activations; state (slots, width) float32, continued and written back.  Returns S * silu(g), (T, width)."""
+    _dev(zxg, state)
+    _need(zxg.dim() == 2 and zxg.stride(1) == 1 and zxg.shape[1] % 3 == 0, "mingru_scan: zxg must be (T, 3 * width)")
+    t, width = zxg.shape[0], zxg.shape[1] // 3
+    _f32c(state, "mingru_scan: state")
+    _need(t == layout.n_tok and state.dim() == 2 and state.shape[1] == width, "mingru_scan: shapes")
+    out = torch.empty((t, width), dtype=zxg.dtype, device=zxg.device)
+    lib = _lib.load()
+    _lib.check(lib.nvx_mingru_scan(_ptr(zxg), zxg.stride(0), _fmt(zxg), _ptr(state), state.shape[0], _ptr(layout.qo_indptr),
+                                   _ptr(layout.pos0), _ptr(layout.state_slot), _ptr(out), t, layout.n_seq, width, _stream()),
+               "nvx_mingru_scan")
+    return out
+
+
+def latent_prep(x, w_q, w_kv, eps: float, slots, cache, heads: int):
+    """After the down projections of latent attention: x (T, q_rank + kv_rank + heads).  Returns (cq, gate): the
+    RMS-normed query latent (T, q_rank) in x's format and sigmoid of the per-head gates (T, heads) float32; the RMS-normed
+    key/value latent of token t is stored at cache[slots[t]] (cache: (slots, kv_rank) in x's format)."""
+    _dev(x, w_q, w_kv, slots, cache)
+    _f32c(w_q, "latent_prep: w_q")
+    _f32c(w_kv, "latent_prep: w_kv")
+    q_rank, kv_rank = w_q.numel(), w_kv.numel()
+    _need(x.dim() == 2 and x.stride(1) == 1 and x.shape[1] == q_rank + kv_rank + heads, "latent_prep: x shape")
+    t = x.shape[0]
+    _need(cache.dtype == x.dtype and cache.is_contiguous() and cache.dim() == 2 and cache.shape[1] == kv_rank, "latent_prep: cache")
+    _need(slots.dtype == torch.int64 and slots.is_contiguous() and slots.numel() == t, "latent_prep: slots must be int64 (T)")
+    cq = torch.empty((t, q_rank), dtype=x.dtype, device=x.device)
+    gate = torch.empty((t, heads), dtype=F32, device=x.device)
+    lib = _lib.load()
+    _lib.check(lib.nvx_latent_prep(_ptr(x), x.stride(0), _fmt(x), _ptr(w_q), _ptr(w_kv), float(eps), _ptr(slots), _ptr(cq), _ptr(cache),
+                                   cache.shape[0], _ptr(gate), t, q_rank, kv_rank, heads, _stream()), "nvx_latent_prep")
+    return cq, gate
+
+
+def latent_attn(q, cache, kv_indices, kv_start, kv_len, layout: StepLayout, scale: float, gate=None):
+    """Attention over cached latents: q (heads, T, rank) folded queries, cache (slots, rank).  Sequence b's tokens are
+    at slots kv_indices[kv_start[b] : kv_start[b] + kv_len[b]]; causal.  Returns (heads, T, rank) in q's format, each
+    head's rows multiplied by gate[t][h] if given."""
+    _dev(q, cache, kv_indices, kv_start, kv_len, gate)
+    _need(q.dim() == 3 and q.is_contiguous(), "latent_attn: q must be contiguous (heads, T, rank)")
+    heads, t, rank = q.shape
+    _need(t == layout.n_tok, "latent_attn: token count")
+    _need(cache.dtype == q.dtype and cache.is_contiguous() and cache.dim() == 2 and cache.shape[1] == rank, "latent_attn: cache")
+    _need(kv_indices.dtype == torch.int32 and kv_indices.is_contiguous(), "latent_attn: kv_indices must be int32")
+    _need(kv_start.dtype == torch.int64 and kv_start.numel() >= layout.n_seq, "latent_attn: kv_start must be int64 (B)")
+    _need(kv_len.dtype == torch.int32 and kv_len.numel() >= layout.n_seq, "latent_attn: kv_len must be int32 (B)")
+    if gate is not None:
+        _f32c(gate, "latent_attn: gate")
+        _need(gate.shape == (t, heads), "latent_attn: gate shape")
+    out = torch.empty_like(q)
+    lib = _lib.load()
+    _lib.check(lib.nvx_latent_attn(_ptr(q), _ptr(cache), _fmt(q), _ptr(kv_indices), _ptr(kv_start), _ptr(kv_len), _ptr(layout.qo_indptr),
+                                   _ptr(layout.tok_seq), _ptr(gate), _ptr(out), heads, rank, t, float(scale), _stream()), "nvx_latent_attn")
+    return out

@@ -57,6 +57,17 @@ _DEFS = {
     "block_table_write_rows": "(Tensor kv_indices, Tensor kv_indptr, Tensor rows, Tensor(a!) table) -> ()",
     "decode_step_setup": "(Tensor step, int stride, int padded_batch, Tensor(a!) table, int pad_start, Tensor(b!) kv_start, "
                          "Tensor(c!) kv_len, Tensor(d!) out_slots, Tensor(e!) positions, Tensor(f!) input_ids, Tensor? prev_ids) -> ()",
+    # layers with a float32 residual stream, per-sequence state and latent attention; the step's layout travels as its four
+    # tensors (qo_indptr and tok_seq absent: one token per sequence)
+    "boundary_norm": "(Tensor m, Tensor w_post, float eps, Tensor? res, Tensor(a!)? hist, int hist_slot, Tensor? mix, Tensor? w_pre, "
+                     "bool pre_f32) -> (Tensor, Tensor?)",
+    "canon_conv": "(Tensor h, Tensor taps, Tensor(a!) state, Tensor pos0, Tensor state_slot, Tensor? qo_indptr, Tensor? tok_seq, "
+                  "ScalarType dtype) -> Tensor",
+    "relu2": "(Tensor x) -> Tensor",
+    "mingru_scan": "(Tensor zxg, Tensor(a!) state, Tensor pos0, Tensor state_slot, Tensor? qo_indptr, Tensor? tok_seq) -> Tensor",
+    "latent_prep": "(Tensor x, Tensor w_q, Tensor w_kv, float eps, Tensor slots, Tensor(a!) cache, int heads) -> (Tensor, Tensor)",
+    "latent_attn": "(Tensor q, Tensor cache, Tensor kv_indices, Tensor kv_start, Tensor kv_len, Tensor pos0, Tensor state_slot, "
+                   "Tensor? qo_indptr, Tensor? tok_seq, float scale, Tensor? gate) -> Tensor",
 }
 for _name, _sig in _DEFS.items():
     _LIB.define(_name + _sig)
@@ -183,6 +194,35 @@ def _decode_step_setup(step, stride, padded_batch, table, pad_start, kv_start, k
                        prev_ids: Optional[torch.Tensor]):
     ops.decode_step_setup(step, stride, padded_batch, table, pad_start, kv_start, kv_len, out_slots, positions, input_ids,
                           prev_ids=prev_ids)
+
+
+def _layout(n_tok, pos0, state_slot, qo_indptr, tok_seq):
+    n_seq = n_tok if qo_indptr is None else qo_indptr.numel() - 1
+    return ops.StepLayout(n_tok, n_seq, pos0, state_slot, qo_indptr, tok_seq)
+
+
+def _boundary_norm(m, w_post, eps, res, hist, hist_slot, mix, w_pre, pre_f32):
+    return ops.boundary_norm(m, w_post, eps, res=res, hist=hist, hist_slot=hist_slot, mix=mix, w_pre=w_pre, pre_f32=pre_f32)
+
+
+def _canon_conv(h, taps, state, pos0, state_slot, qo_indptr, tok_seq, dtype):
+    return ops.canon_conv(h, taps, state, _layout(h.shape[0], pos0, state_slot, qo_indptr, tok_seq), dtype)
+
+
+def _relu2(x):
+    return ops.relu2(x)
+
+
+def _mingru_scan(zxg, state, pos0, state_slot, qo_indptr, tok_seq):
+    return ops.mingru_scan(zxg, state, _layout(zxg.shape[0], pos0, state_slot, qo_indptr, tok_seq))
+
+
+def _latent_prep(x, w_q, w_kv, eps, slots, cache, heads):
+    return ops.latent_prep(x, w_q, w_kv, eps, slots, cache, heads)
+
+
+def _latent_attn(q, cache, kv_indices, kv_start, kv_len, pos0, state_slot, qo_indptr, tok_seq, scale, gate):
+    return ops.latent_attn(q, cache, kv_indices, kv_start, kv_len, _layout(q.shape[1], pos0, state_slot, qo_indptr, tok_seq), scale, gate)
 
 
 for _name in _DEFS:

@@ -108,7 +108,8 @@ def test_every_kernel_entry_point_has_a_custom_op():
              "nvx_decode_step_setup": "decode_step_setup", "nvx_peer_allreduce_norm": "peer_allreduce_norm",
              "nvx_sample_shard": "sample_shard", "nvx_sample_pick": "sample_pick", "nvx_lmhead_pack": "lmhead_pack",
              "nvx_lmhead_sample": "lmhead_sample", "nvx_linear_stream": "linear_stream", "nvx_splitk_sum": "splitk_sum",
-             "nvx_linear_block": "linear_block"}
+             "nvx_linear_block": "linear_block", "nvx_boundary_norm": "boundary_norm", "nvx_canon_conv": "canon_conv", "nvx_relu2": "relu2",
+             "nvx_mingru_scan": "mingru_scan", "nvx_latent_prep": "latent_prep", "nvx_latent_attn": "latent_attn"}
     helpers = {"nvx_abi_version", "nvx_last_error", "nvx_linear_decode_splits", "nvx_decode_plan_ws_ints", "nvx_decode_partial_ws_floats",
                "nvx_prefill_plan_ws_ints", "nvx_sample_ws_bytes", "nvx_paged_decode_noalloc_max_batch",
                "nvx_lmhead_max_rows", "nvx_lmhead_rows_per_pass", "nvx_lmhead_packed_elems", "nvx_lmhead_ws_bytes",
