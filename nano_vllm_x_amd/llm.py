@@ -47,8 +47,8 @@ class LLM:
                  pp_size: int = 1, nccl_port: int = 29500, device_ids: Optional[list] = None,
                  enforce_eager: bool = False, context_len: int = 2048, kv_cache_size: Optional[int] = None, seed: int = 0,
                  prefix_reuse: bool = False, max_prefill_tokens: Optional[int] = None, stop_at_context_len: bool = False,
-                 chunked_prefill: bool = False, run_ahead: bool = False):
-        kwargs = dict(model=model, gpu_memory_utilization=gpu_memory_utilization, max_bs=max_bs, tp_size=tp_size, pp_size=pp_size,
+                 chunked_prefill: bool = False, run_ahead: bool = False, dtype: Optional[str] = None):
+        kwargs = dict(dtype=dtype, model=model, gpu_memory_utilization=gpu_memory_utilization, max_bs=max_bs, tp_size=tp_size, pp_size=pp_size,
                       nccl_port=nccl_port, device_ids=device_ids, enforce_eager=enforce_eager, context_len=context_len,
                       kv_cache_size=kv_cache_size, seed=seed, prefix_reuse=prefix_reuse, max_prefill_tokens=max_prefill_tokens,
                       stop_at_context_len=stop_at_context_len, chunked_prefill=chunked_prefill, run_ahead=run_ahead)

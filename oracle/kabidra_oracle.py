@@ -10,8 +10,6 @@ layers 0..i.
 """
 from __future__ import annotations
 
-import math
-
 import torch
 
 
@@ -28,10 +26,6 @@ def norm_plain(v, w, eps):
     return rms(v, eps) * w
 
 
-def gelu_tanh(z):
-    return 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
-
-
 def canon(h: torch.Tensor, k: torch.Tensor) -> torch.Tensor:
     """h (tokens, width) of ONE sequence from its first token; k (width, taps).  Returns h + causal convolution."""
     taps = k.shape[1]
@@ -44,19 +38,23 @@ def canon(h: torch.Tensor, k: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def mingru(h: torch.Tensor, p: dict) -> torch.Tensor:
-    """minGRU layer (gates from the current token alone) with its projections; h (tokens, width) of one sequence from its start."""
-    z = torch.sigmoid(h @ p["z"].T + p["z.b"])
-    u = h @ p["x"].T + p["x.b"]
+def gru_scan(z_pre: torch.Tensor, u: torch.Tensor, g_pre: torch.Tensor, s0=None):
+    """The recurrence alone, from pre-activations (tokens, n): returns (outputs before the output projection, last state)."""
+    z = torch.sigmoid(z_pre)
     cand = torch.where(u >= 0, u + 0.5, torch.sigmoid(u))
-    gate = h @ p["g"].T
-    gate = gate * torch.sigmoid(gate)
-    s = torch.zeros(p["z"].shape[0], dtype=h.dtype)
+    gate = g_pre * torch.sigmoid(g_pre)
+    s = torch.zeros(z.shape[1], dtype=z.dtype) if s0 is None else s0.clone()
     ys = []
-    for t in range(h.shape[0]):
+    for t in range(z.shape[0]):
         s = (1.0 - z[t]) * s + z[t] * cand[t]
         ys.append(s * gate[t])
-    return torch.stack(ys) @ p["o"].T
+    return torch.stack(ys), s
+
+
+def mingru(h: torch.Tensor, p: dict) -> torch.Tensor:
+    """minGRU layer (gates from the current token alone) with its projections; h (tokens, width) of one sequence from its start."""
+    y, _ = gru_scan(h @ p["z"].T + p["z.b"], h @ p["x"].T + p["x.b"], h @ p["g"].T)
+    return y @ p["o"].T
 
 
 def latent_attention(h: torch.Tensor, p: dict, m: dict, eps: float) -> torch.Tensor:
