@@ -366,8 +366,159 @@ def cpu_baseline(prompts, max_tokens, n_req: int, new_tokens: int, gpu_config1_t
 
 
 # ---------------------------------------------------------------------------------------------------
+# --arch-compare: Kabidra (minGRU + latent attention) beside Qwen3 at equal width, depth, feed-forward and vocabulary
+# ---------------------------------------------------------------------------------------------------
+ARCH_SIZES = {   # name -> width, layers, ff, heads (head size 128 in both models), latent ranks, vocabulary
+    "w1024": dict(width=1024, layers=6, ff=3072, heads=16, q_rank=512, kv_rank=256, vocab=32000),
+    "w2048": dict(width=2048, layers=6, ff=6144, heads=16, q_rank=768, kv_rank=512, vocab=32000),
+    "w4096": dict(width=4096, layers=3, ff=12288, heads=32, q_rank=1536, kv_rank=512, vocab=32000),
+}
+
+
+def _kabidra_config(z):
+    att = {"type": "latent_attention", "mixer": {"heads": z["heads"], "dim": 128, "vdim": 128, "q_rank": z["q_rank"], "kv_rank": z["kv_rank"],
+                                                 "scale": 128 ** -0.5}, "mlp": {"kind": "dense", "ff": z["ff"]}}
+    gru = {"type": "mingru", "mixer": {"width": z["width"]}, "mlp": {"kind": "dense", "ff": z["ff"]}}
+    return {"architecture": "Kabidra", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-5}, "canon": {"taps": 4},
+            "layers": [att if i % 3 == 2 else gru for i in range(z["layers"])]}
+
+
+def _qwen3_config(z):
+    return {"architectures": ["Qwen3ForCausalLM"], "vocab_size": z["vocab"], "hidden_size": z["width"], "intermediate_size": z["ff"],
+            "num_hidden_layers": z["layers"], "num_attention_heads": z["heads"], "num_key_value_heads": 8, "head_dim": 128,
+            "tie_word_embeddings": False, "torch_dtype": "bfloat16"}
+
+
+def _serve_once(path, n_seq, prompt_len, new_tokens, eager):
+    """Prefill and decode rates of one engine on n_seq prompts of prompt_len tokens, new_tokens decoded each."""
+    from nano_vllm_x_amd.core.common import SamplingParams
+    from nano_vllm_x_amd.core.engine import Engine
+
+    eng = Engine(model=path, gpu_memory_utilization=0.5, max_bs=n_seq, enforce_eager=eager, context_len=prompt_len + new_tokens + 8,
+                 kv_cache_size=n_seq * (prompt_len + new_tokens + 8))
+    rnd = random.Random(0)
+    out = {}
+    for rep in range(2):       # the first pass warms up (library handles, allocator); the second is reported
+        s0 = dict(eng.model_runner.stats)
+        for i in range(n_seq):
+            eng.add_sequence(f"p{rep}_{i}", [rnd.randrange(0, 30000) for _ in range(prompt_len)],
+                             SamplingParams(temperature=0.0, ignore_eos=True, max_new_tokens=new_tokens))
+        while eng.has_unfinished_sequences():
+            eng.step()
+        s1 = eng.model_runner.stats
+        pre, dec = s1["prefill_s"] - s0["prefill_s"], s1["decode_s"] - s0["decode_s"]
+        out = {"prefill_tokens_per_s": round(n_seq * prompt_len / pre), "decode_tokens_per_s": round(n_seq * (new_tokens - 1) / dec),
+               "prefill_ms": round(pre * 1e3, 2), "decode_step_ms": round(dec * 1e3 / (new_tokens - 1), 3),
+               "decode": "hipGraph" if s1["graph_steps"] - s0["graph_steps"] else "eager"}
+    eng.shutdown()
+    del eng
+    torch.cuda.empty_cache()
+    return out
+
+
+def _time_us(fn, reps=20):
+    fn()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(reps):
+        fn()
+    b.record()
+    b.synchronize()
+    return a.elapsed_time(b) * 1e3 / reps
+
+
+def _kernel_table(z, t_pre, n_dec, ctx):
+    """Each kernel of the new design beside the like kernel of Qwen3 at the same shape: time, and the fraction of its
+    roofline (HBM bytes it must move at 8 TB/s; attention in prefill: its multiply-adds at the dense bf16 MFMA peak)."""
+    from nano_vllm_x_amd import ops
+    dev, bf = torch.device("cuda"), torch.bfloat16
+    w, ff, h, r = z["width"], z["ff"], z["heads"], z["kv_rank"]
+    rows = []
+
+    def layout(n_seq, q_len, pos0):
+        p = torch.full((n_seq,), pos0, dtype=torch.int64, device=dev)
+        sl = torch.arange(n_seq, dtype=torch.int32, device=dev)
+        if q_len == 1:
+            return ops.StepLayout(n_seq, n_seq, p, sl)
+        qo = torch.arange(0, n_seq + 1, dtype=torch.int32, device=dev) * q_len
+        return ops.StepLayout(n_seq * q_len, n_seq, p, sl, qo, torch.arange(n_seq, dtype=torch.int32, device=dev).repeat_interleave(q_len))
+
+    def add(name, phase, us, bytes_=None, flops=None, like=None):
+        frac = (bytes_ / (us * 1e-6) / (HBM_PEAK_GBS * 1e9)) if bytes_ else (flops / (us * 1e-6) / (MFMA_BF16_PEAK_TFLOPS * 1e12))
+        rows.append({"kernel": name, "phase": phase, "us": round(us, 1), "of_roofline": round(frac, 3), "bound": "HBM" if bytes_ else "MFMA",
+                     "like": like})
+
+    for phase, (n_seq, q_len, pos0) in (("prefill", (t_pre // 1024, 1024, 0)), ("decode", (n_dec, 1, ctx))):
+        t = n_seq * q_len
+        lay = layout(n_seq, q_len, pos0)
+        m, res = torch.randn(t, w, device=dev).to(bf), torch.randn(t, w, device=dev)
+        wv = torch.zeros(w, device=dev)
+        # sublayer boundary: reads m (2 B) and the stream (4 B), writes the stream (4 B) and the normed rows (4 B)
+        add("boundary_norm", phase, _time_us(lambda: ops.boundary_norm(m, wv, 1e-5, res=res, w_pre=wv)), bytes_=t * w * 14, like="rmsnorm+residual")
+        resb = res.to(bf)
+        add("qwen3 rmsnorm+residual", phase, _time_us(lambda: ops.rmsnorm(m, wv.to(bf), 1e-5, resb)), bytes_=t * w * 8)
+        st = torch.zeros(n_seq + 1, 3, w, device=dev)
+        taps = torch.randn(w, 4, device=dev)
+        add("canon_conv", phase, _time_us(lambda: ops.canon_conv(res, taps, st, lay, bf)), bytes_=t * w * 6 + n_seq * 3 * w * 8, like="(none)")
+        zxg = torch.randn(t, 3 * w, device=dev).to(bf)
+        gs = torch.zeros(n_seq + 1, w, device=dev)
+        add("mingru_scan", phase, _time_us(lambda: ops.mingru_scan(zxg, gs, lay)), bytes_=t * w * 8 + n_seq * w * 8, like="silu_mul")
+        up = torch.randn(t, ff, device=dev).to(bf)
+        add("relu2", phase, _time_us(lambda: ops.relu2(up)), bytes_=t * ff * 4, like="silu_mul")
+        gu = torch.randn(t, 2 * ff, device=dev).to(bf)
+        add("qwen3 silu_mul", phase, _time_us(lambda: ops.silu_mul(gu)), bytes_=t * ff * 6)
+        # latent attention over a cache of (tokens, kv_rank)
+        kv_len = pos0 + q_len
+        pool = torch.randn(n_seq * kv_len, r, device=dev).to(bf)
+        idx = torch.arange(n_seq * kv_len, dtype=torch.int32, device=dev)
+        kv_start = torch.arange(n_seq, dtype=torch.int64, device=dev) * kv_len
+        kvl = torch.full((n_seq,), kv_len, dtype=torch.int32, device=dev)
+        q = torch.randn(h, t, r, device=dev).to(bf)
+        us = _time_us(lambda: ops.latent_attn(q, pool, idx, kv_start, kvl, lay, 0.1), reps=3 if phase == "prefill" else 20)
+        if phase == "prefill":
+            pairs = n_seq * q_len * (q_len + 1) // 2
+            add("latent_attn", phase, us, flops=4.0 * h * r * pairs, like="paged_prefill")
+        else:
+            add("latent_attn", phase, us, bytes_=n_seq * kv_len * r * 2 + 2 * t * h * r * 2, like="paged_decode")
+    return rows
+
+
+def arch_compare(args):
+    import tempfile
+
+    torch.cuda.set_device(0)
+    result = {"metric": "prefill and decode tokens/s, Kabidra beside Qwen3 at equal width, depth, feed-forward and vocabulary",
+              "dtype": "bf16", "data": "synthetic (random token ids, random-init weights)", "n_gpus": 1,
+              "workload": {"prefill": f"{args.arch_seqs} prompts of {args.arch_prompt} tokens in one step",
+                           "decode": f"{args.arch_seqs} sequences, {args.arch_new} steps from context {args.arch_prompt}"},
+              "sizes": {}}
+    for name in args.arch_sizes.split(","):
+        z = ARCH_SIZES[name]
+        entry = {"geometry": z}
+        with tempfile.TemporaryDirectory() as tmp:
+            for model, cfg in (("kabidra", _kabidra_config(z)), ("qwen3", _qwen3_config(z))):
+                d = os.path.join(tmp, model)
+                os.makedirs(d)
+                with open(os.path.join(d, "config.json"), "w") as f:
+                    json.dump(cfg, f)
+                entry[model] = _serve_once(d, args.arch_seqs, args.arch_prompt, args.arch_new, args.enforce_eager)
+                print(f"[arch-compare] {name} {model}: {entry[model]}", file=sys.stderr, flush=True)
+        with torch.inference_mode():
+            entry["kernels"] = _kernel_table(z, args.arch_seqs * args.arch_prompt, args.arch_seqs, args.arch_prompt)
+        result["sizes"][name] = entry
+    print(json.dumps(result), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
+    ap.add_argument("--arch-compare", action="store_true",
+                    help="instead of the headline workload: prefill and decode rates of Kabidra beside Qwen3 at equal sizes, and "
+                         "each of its kernels beside the like Qwen3 kernel against its roofline (one JSON line)")
+    ap.add_argument("--arch-sizes", default="w1024,w2048,w4096")
+    ap.add_argument("--arch-seqs", type=int, default=16)
+    ap.add_argument("--arch-prompt", type=int, default=1024)
+    ap.add_argument("--arch-new", type=int, default=33)
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2)
     ap.add_argument("--warmup", type=int, default=1)
@@ -389,6 +540,8 @@ def main():
     ap.add_argument("--cpu-new-tokens", type=int, default=48)
     ap.add_argument("--roofline-every", type=int, default=8)
     args = ap.parse_args()
+    if args.arch_compare:
+        return arch_compare(args)
 
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:
         # typed plainly (`python3 bench.py --gpus N`): start the N ranks as a fresh child job -- this process has made
