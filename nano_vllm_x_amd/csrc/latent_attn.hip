@@ -159,6 +159,188 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(
     }
 }
 
+// ---- the same on the matrix cores (16-bit formats, rank a multiple of 32, at most 512) -----------------------------------
+// One workgroup per (query token, group of 16 heads); its four waves take every fourth tile of 16 keys and merge at the
+// end.  Per tile:
+//   S^T (16 keys x 16 heads) = C_tile (16 x rank) . Q~^T (rank x 16)        v_mfma_f32_16x16x32, rank / 32 of them; the A
+//       operand is read straight from the cache rows (lane (key, quarter) takes 16 bytes per k-step) and parked in LDS;
+//   the result leaves every lane with one head (lane & 15) and four keys (4 * quarter + r): the running maximum and sum of
+//       a head are kept per lane, reduced over the quarters where needed;
+//   O^T (rank x 16 heads) += C_tile^T (rank x 16 keys) . P^T (16 keys x 16 heads)   v_mfma_f32_16x16x16, 32 columns a pair:
+//       the pair's A operands are the even and the odd columns, so one 4-byte LDS read (key 4 * quarter + r, columns
+//       2 i and 2 i + 1 of the 32) feeds both; P^T is exactly what the lane holds.  The weights stay float32 up to here
+//       and enter as hi + lo (two products), which keeps 16 bits of their mantissa.
+// Scores, maximum, exponentials and sums are float32.
+typedef __attribute__((ext_vector_type(4))) short la_s16x4;
+typedef __attribute__((ext_vector_type(8))) __bf16 la_bf16x8;
+typedef __attribute__((ext_vector_type(8))) _Float16 la_f16x8;
+typedef __attribute__((ext_vector_type(4))) _Float16 la_f16x4;
+
+template <typename A> __device__ __forceinline__ nvx_f32x4 la_mfma32(nvx_u32x4 a, nvx_u32x4 b, nvx_f32x4 c) {
+    if constexpr (sizeof(A) == 2 && __is_same(A, __bf16))
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(la_bf16x8, a), __builtin_bit_cast(la_bf16x8, b), c, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(la_f16x8, a), __builtin_bit_cast(la_f16x8, b), c, 0, 0, 0);
+}
+template <typename A> __device__ __forceinline__ nvx_f32x4 la_mfma16(uint2 a, uint2 b, nvx_f32x4 c) {
+    if constexpr (__is_same(A, __bf16))
+        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(la_s16x4, a), __builtin_bit_cast(la_s16x4, b), c, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(la_f16x4, a), __builtin_bit_cast(la_f16x4, b), c, 0, 0, 0);
+}
+template <typename A> __device__ __forceinline__ uint32_t la_pack2(float lo, float hi) {
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    typedef A a2 __attribute__((ext_vector_type(2)));
+    const f2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, a2));
+}
+template <typename A> __device__ __forceinline__ float la_round(float v) { return (float)(A)v; }
+
+#define LA_PAD 8     // elements between the rows of a parked tile: 16-byte rows, and the four quarters hit different banks
+
+template <typename A, int RKM>      // RKM: k-steps of 32 the registers are sized for (rank <= 32 * RKM)
+__global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
+    const A* __restrict__ q, const A* __restrict__ cache, const int32_t* __restrict__ kv_indices, const int64_t* __restrict__ kv_start,
+    const int32_t* __restrict__ kv_len, const int32_t* __restrict__ qo_indptr, const int32_t* __restrict__ tok_seq,
+    const float* __restrict__ gate, A* __restrict__ out, int heads, int rank, int64_t n_tok, float scale) {
+    extern __shared__ float lds[];
+    constexpr int NB2 = RKM;                   // pairs of 16-column blocks = rank / 32
+    const int steps = rank >> 5;
+    const int64_t t = blockIdx.x;
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, l16 = lane & 15, quarter = lane >> 4;
+    const int head = blockIdx.y * 16 + l16;
+    const int b = tok_seq ? tok_seq[t] : (int)t;
+    const int64_t q0 = qo_indptr ? qo_indptr[b] : t;
+    const int64_t q_len = qo_indptr ? qo_indptr[b + 1] - q0 : 1;
+    const int64_t n_keys = (int64_t)kv_len[b] - q_len + (t - q0) + 1;
+    const int32_t* idx = kv_indices + kv_start[b];
+    const int row_elems = rank + LA_PAD;
+    uint16_t* tile = reinterpret_cast<uint16_t*>(lds) + (size_t)wv * 16 * row_elems;     // this wave's parked tile
+
+    nvx_u32x4 qb[RKM];
+#pragma unroll
+    for (int ks = 0; ks < RKM; ++ks) {
+        qb[ks] = nvx_u32x4{0u, 0u, 0u, 0u};
+        if (ks < steps && head < heads)
+            qb[ks] = *reinterpret_cast<const nvx_u32x4*>(q + ((int64_t)head * n_tok + t) * rank + 32 * ks + 8 * quarter);
+    }
+    nvx_f32x4 o_acc[2 * NB2];
+#pragma unroll
+    for (int i = 0; i < 2 * NB2; ++i) o_acc[i] = nvx_f32x4{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;      // of head l16; l_run: this quarter's keys only
+
+    const int64_t n_tiles = (n_keys + 15) >> 4;
+    for (int64_t j = wv; j < n_tiles; j += 4) {
+        const int64_t key = j * 16 + l16;
+        const int slot = idx[key < n_keys ? key : 0];            // a key past the end reads a real row and is masked below
+        const A* row = cache + (int64_t)slot * rank;
+        nvx_f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < RKM; ++ks) {
+            if (ks < steps) {
+                const nvx_u32x4 a = *reinterpret_cast<const nvx_u32x4*>(row + 32 * ks + 8 * quarter);
+                *reinterpret_cast<nvx_u32x4*>(tile + l16 * row_elems + 32 * ks + 8 * quarter) = a;
+                sacc = la_mfma32<A>(a, qb[ks], sacc);
+            }
+        }
+        // the tile is parked before any lane reads it back transposed (one wave: its LDS operations complete in order)
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        float sv[4], mx = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            sv[r] = (j * 16 + 4 * quarter + r) < n_keys ? sacc[r] * scale : -INFINITY;
+            mx = fmaxf(mx, sv[r]);
+        }
+        mx = fmaxf(mx, xor16(mx));
+        mx = fmaxf(mx, xor32(mx));
+        const float m_new = fmaxf(m_run, mx);                    // finite: a tile has at least one visible key
+        const float alpha = __expf(m_run - m_new);
+        m_run = m_new;
+        l_run *= alpha;
+        float p[4], ph[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            p[r] = __expf(sv[r] - m_new);
+            l_run += p[r];
+            ph[r] = la_round<A>(p[r]);
+        }
+        const uint2 p_hi = make_uint2(la_pack2<A>(ph[0], ph[1]), la_pack2<A>(ph[2], ph[3]));
+        const uint2 p_lo = make_uint2(la_pack2<A>(p[0] - ph[0], p[1] - ph[1]), la_pack2<A>(p[2] - ph[2], p[3] - ph[3]));
+        const uint32_t* tile32 = reinterpret_cast<const uint32_t*>(tile);
+#pragma unroll
+        for (int b2 = 0; b2 < NB2; ++b2) {
+            if (b2 < steps) {
+                uint32_t d[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) d[r] = tile32[((4 * quarter + r) * row_elems + 32 * b2) / 2 + l16];
+                const uint2 even = make_uint2((d[0] & 0xffffu) | (d[1] << 16), (d[2] & 0xffffu) | (d[3] << 16));
+                const uint2 odd = make_uint2((d[0] >> 16) | (d[1] & 0xffff0000u), (d[2] >> 16) | (d[3] & 0xffff0000u));
+                o_acc[2 * b2] *= alpha;
+                o_acc[2 * b2 + 1] *= alpha;
+                o_acc[2 * b2] = la_mfma16<A>(even, p_hi, o_acc[2 * b2]);
+                o_acc[2 * b2] = la_mfma16<A>(even, p_lo, o_acc[2 * b2]);
+                o_acc[2 * b2 + 1] = la_mfma16<A>(odd, p_hi, o_acc[2 * b2 + 1]);
+                o_acc[2 * b2 + 1] = la_mfma16<A>(odd, p_lo, o_acc[2 * b2 + 1]);
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");      // the reads are done before the next tile is parked
+    }
+
+    // merge the four waves' partial results: 2 and 3 into 0 and 1, then 1 into 0.  Every lane parks its own values; the lane
+    // of the same number in the other wave holds the same head and columns.
+    const int vals = 8 * steps + 2;
+    auto park = [&](int region) {
+        float* base = lds + (size_t)region * vals * 64 + lane;
+#pragma unroll
+        for (int i = 0; i < 2 * NB2; ++i)
+            if (i < 2 * steps) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) base[(4 * i + r) * 64] = o_acc[i][r];
+            }
+        base[(8 * steps) * 64] = m_run;
+        base[(8 * steps + 1) * 64] = l_run;
+    };
+    auto take = [&](int region) {
+        const float* base = lds + (size_t)region * vals * 64 + lane;
+        const float m_o = base[(8 * steps) * 64], l_o = base[(8 * steps + 1) * 64];
+        const float m_new = fmaxf(m_run, m_o);
+        const float ref = m_new == -INFINITY ? 0.f : m_new;
+        const float fa = __expf(m_run - ref), fb = __expf(m_o - ref);
+        m_run = m_new;
+        l_run = l_run * fa + l_o * fb;
+#pragma unroll
+        for (int i = 0; i < 2 * NB2; ++i)
+            if (i < 2 * steps) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) o_acc[i][r] = o_acc[i][r] * fa + base[(4 * i + r) * 64] * fb;
+            }
+    };
+    __syncthreads();                 // every wave is done with its tile: the memory changes hands
+    if (wv >= 2) park(wv - 2);
+    __syncthreads();
+    if (wv < 2) take(wv);
+    __syncthreads();
+    if (wv == 1) park(0);
+    __syncthreads();
+    if (wv != 0) return;
+    take(0);
+    float l_tot = l_run + xor16(l_run);
+    l_tot += xor32(l_tot);
+    if (head >= heads) return;
+    const float f = (gate ? gate[t * heads + head] : 1.0f) / l_tot;
+    A* orow = out + ((int64_t)head * n_tok + t) * rank;
+#pragma unroll
+    for (int b2 = 0; b2 < NB2; ++b2) {
+        if (b2 < steps) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {        // row i = 4 * quarter + r of the pair's blocks: columns 2 i (even) and 2 i + 1 (odd)
+                const int c = 32 * b2 + 2 * (4 * quarter + r);
+                *reinterpret_cast<uint32_t*>(orow + c) = la_pack2<A>(o_acc[2 * b2][r] * f, o_acc[2 * b2 + 1][r] * f);
+            }
+        }
+    }
+}
+
 template <typename A>
 static void launch_prep(const void* x, int64_t x_stride, const float* w_q, const float* w_kv, float eps, const int64_t* slots, void* cq,
                         void* cache, int64_t n_slots, float* gate, int64_t n_tok, int q_rank, int kv_rank, int heads, hipStream_t s) {
@@ -170,6 +352,22 @@ template <typename A>
 static void launch_attn(const void* q, const void* cache, const int32_t* kv_indices, const int64_t* kv_start, const int32_t* kv_len,
                         const int32_t* qo_indptr, const int32_t* tok_seq, const float* gate, void* out, int heads, int rank, int64_t n_tok,
                         float scale, hipStream_t s) {
+    if constexpr (sizeof(A) == 2) {
+        if (rank % 32 == 0 && rank <= 512 && nvx_aligned16(q) && nvx_aligned16(cache) && nvx_aligned16(out) && n_tok <= 0x7fffffff) {
+            const int steps = rank / 32;
+            const size_t tiles = (size_t)4 * 16 * (rank + LA_PAD) * 2, merge = (size_t)2 * (8 * steps + 2) * 64 * 4;
+            const size_t lds = tiles > merge ? tiles : merge;
+            const dim3 grid((unsigned)n_tok, (unsigned)((heads + 15) / 16));
+#define NVX_LA_MFMA(RKM)                                                                                                            \
+    hipLaunchKernelGGL((latent_attn_mfma_kernel<A, RKM>), grid, dim3(256), lds, s, (const A*)q, (const A*)cache, kv_indices, kv_start, \
+                       kv_len, qo_indptr, tok_seq, gate, (A*)out, heads, rank, n_tok, scale)
+            if (steps <= 4) NVX_LA_MFMA(4);
+            else if (steps <= 8) NVX_LA_MFMA(8);
+            else NVX_LA_MFMA(16);
+#undef NVX_LA_MFMA
+            return;
+        }
+    }
     constexpr int HG = 4;
     const size_t lds = (size_t)(HG * rank + LA_KT * HG + LA_KT + 4 * HG) * 4;
     hipLaunchKernelGGL((latent_attn_kernel<A, HG>), dim3((unsigned)n_tok, (unsigned)((heads + HG - 1) / HG)), dim3(256), lds, s,

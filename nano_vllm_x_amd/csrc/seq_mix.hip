@@ -17,6 +17,16 @@ namespace NVX_NS {
 template <typename A> __device__ __forceinline__ float ldf(const A* p, int64_t i) { return (float)p[i]; }
 template <typename A> __device__ __forceinline__ void stf(A* p, int64_t i, float v) { p[i] = (A)v; }
 
+// four consecutive elements at once (the caller guarantees a multiple-of-4 offset into a 16-byte-aligned row)
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+template <typename A> struct vec4 { typedef A type __attribute__((ext_vector_type(4))); };
+template <typename A> __device__ __forceinline__ f32x4v ld4(const A* p) {
+    return __builtin_convertvector(*reinterpret_cast<const typename vec4<A>::type*>(p), f32x4v);
+}
+template <typename A> __device__ __forceinline__ void st4(A* p, f32x4v v) {
+    *reinterpret_cast<typename vec4<A>::type*>(p) = __builtin_convertvector(v, typename vec4<A>::type);
+}
+
 // sum over a workgroup of 256 threads; every thread gets the total.  `red` holds 4 floats; safe to call repeatedly.
 __device__ __forceinline__ float block_sum256(float v, float* red) {
     v = wave_sum(v);
@@ -69,6 +79,57 @@ __global__ __launch_bounds__(256) void boundary_norm_kernel(
     }
 }
 
+// The same, for rows of at most 256 * 4 * VPT values with a multiple of 4 of them: every thread keeps its part of the row
+// in registers, so m and the stream are read once and written once.
+template <typename A, int VPT>
+__global__ __launch_bounds__(256) void boundary_norm_reg_kernel(
+    const A* __restrict__ m, int64_t m_stride, const float* __restrict__ res, const float* __restrict__ w_post,
+    float* __restrict__ hist, int64_t hist_stride, int hist_slot, int n_mix, const float* __restrict__ mix,
+    float* __restrict__ x_out, const float* __restrict__ w_pre, float* __restrict__ y_f32, A* __restrict__ y_act,
+    int width, float eps) {
+    __shared__ float red[4];
+    const int64_t t = blockIdx.x;
+    const A* mr = m + t * m_stride;
+    const int64_t row = t * (int64_t)width;
+    f32x4v v[VPT];
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+        const int c = (threadIdx.x + k * 256) * 4;
+        v[k] = c < width ? ld4(mr + c) : f32x4v{0.f, 0.f, 0.f, 0.f};
+        ss += v[k].x * v[k].x + v[k].y * v[k].y + v[k].z * v[k].z + v[k].w * v[k].w;
+    }
+    const float r_post = 1.0f / sqrtf(block_sum256(ss, red) / (float)width + eps);
+    float ss2 = 0.f;
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+        const int c = (threadIdx.x + k * 256) * 4;
+        if (c >= width) continue;
+        f32x4v r = v[k] * r_post * (1.0f + *reinterpret_cast<const f32x4v*>(w_post + c));
+        if (res) r += *reinterpret_cast<const f32x4v*>(res + row + c);
+        if (hist_slot >= 0) *reinterpret_cast<f32x4v*>(hist + (int64_t)hist_slot * hist_stride + row + c) = r;
+        f32x4v x = r;
+        if (n_mix > 0) {
+            x = f32x4v{0.f, 0.f, 0.f, 0.f};
+            for (int j = 0; j < n_mix; ++j)
+                x += mix[j] * (j == hist_slot ? r : *reinterpret_cast<const f32x4v*>(hist + (int64_t)j * hist_stride + row + c));
+        }
+        *reinterpret_cast<f32x4v*>(x_out + row + c) = x;
+        v[k] = x;
+        ss2 += x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w;
+    }
+    if (!w_pre) return;
+    const float r_pre = 1.0f / sqrtf(block_sum256(ss2, red) / (float)width + eps);
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+        const int c = (threadIdx.x + k * 256) * 4;
+        if (c >= width) continue;
+        const f32x4v y = v[k] * r_pre * (1.0f + *reinterpret_cast<const f32x4v*>(w_pre + c));
+        if (y_f32) *reinterpret_cast<f32x4v*>(y_f32 + row + c) = y;
+        else st4(y_act + row + c, y);
+    }
+}
+
 // ---- canon: h + causal convolution over time, per channel -----------------------------------------------------------
 // taps[c][j] multiplies the input (taps_n - 1 - j) tokens back.  state[slot][r] (r < taps_n - 1) is the input at position
 // pos0 - (taps_n - 1) + r.
@@ -98,6 +159,35 @@ __global__ __launch_bounds__(256) void canon_conv_kernel(
         }
         stf(out, id, acc);
     }
+}
+
+// The same with four channels per thread (width a multiple of 4): workgroup (x, t) takes 1024 channels of token t.
+template <typename A>
+__global__ __launch_bounds__(256) void canon_conv_vec_kernel(
+    const float* __restrict__ h, const float* __restrict__ taps, int taps_n, const float* __restrict__ state,
+    const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ qo_indptr, const int64_t* __restrict__ pos0,
+    const int32_t* __restrict__ state_slot, A* __restrict__ out, int width) {
+    const int64_t t = blockIdx.y;
+    const int c = (blockIdx.x * 256 + threadIdx.x) * 4;
+    if (c >= width) return;
+    const int b = tok_seq ? tok_seq[t] : (int)t;
+    const int slot = state_slot[b];
+    if (slot < 0) { st4(out + t * width + c, f32x4v{0.f, 0.f, 0.f, 0.f}); return; }
+    const int64_t q0 = qo_indptr ? qo_indptr[b] : t;
+    const int64_t local = t - q0;
+    const bool has_state = pos0[b] > 0;
+    const int hist_n = taps_n - 1;
+    f32x4v acc = *reinterpret_cast<const f32x4v*>(h + t * width + c);
+    for (int j = 0; j < taps_n; ++j) {
+        const int64_t s = local - hist_n + j;
+        f32x4v v;
+        if (s >= 0) v = *reinterpret_cast<const f32x4v*>(h + (q0 + s) * width + c);
+        else if (has_state) v = *reinterpret_cast<const f32x4v*>(state + ((int64_t)slot * hist_n + (hist_n + s)) * width + c);
+        else continue;
+        const float* tp = taps + (int64_t)c * taps_n + j;
+        acc += f32x4v{tp[0], tp[taps_n], tp[2 * taps_n], tp[3 * taps_n]} * v;
+    }
+    st4(out + t * width + c, acc);
 }
 
 // After the convolution has read the old tail: the last taps_n - 1 inputs of every sequence become its new tail.
@@ -136,63 +226,98 @@ __global__ __launch_bounds__(256) void relu2_kernel(const A* __restrict__ x, A* 
 // ---- minGRU ---------------------------------------------------------------------------------------------------------
 // zxg[t] = [ z pre-activation | candidate pre-activation u | output-gate pre-activation g ], `width` each.
 //   z = sigmoid(.),  cand = u + 1/2 (u >= 0) or sigmoid(u) (u < 0),  S <- (1 - z) S + z cand,  out = S * silu(g)
-// The recurrence is S_t = a_t S_(t-1) + b_t with a = 1 - z, b = z cand.  A workgroup takes 64 channels of one sequence
-// and walks its tokens in rounds of SEG * 4 tokens: each of its 4 waves scans SEG consecutive tokens from a zero
-// state (keeping the running product of a), the four partial results are chained through LDS, and every wave then adds
-// its incoming state times the running product.  All of it in float32.
+// The recurrence is S_t = a_t S_(t-1) + b_t with a = 1 - z, b = z cand: segments of the time axis are scanned in parallel
+// and chained.  All of it in float32.
 __device__ __forceinline__ float sigmoidf_(float v) { return 1.0f / (1.0f + expf(-v)); }
+// 16-bit activation formats: the hardware exponential (relative error ~1e-6, far below the format's own rounding)
+template <typename A> __device__ __forceinline__ float sigm(float v) {
+    if constexpr (sizeof(A) == 4) return 1.0f / (1.0f + expf(-v));
+    else return 1.0f / (1.0f + __expf(-v));
+}
+
+// A workgroup takes GRU_CB channels of one sequence and walks its tokens in rounds of GRU_NSEG * SEG tokens: thread
+// (segment, channel pair) scans SEG consecutive tokens from a zero state, keeping the running product of a; the segments'
+// results are chained through LDS, and every thread then adds its incoming state times the running product.
+#define GRU_CB 32        // channels per workgroup (16 lanes x 2)
+#define GRU_NSEG 16      // time segments per round
 
 template <typename A, int SEG>
 __global__ __launch_bounds__(256) void mingru_scan_kernel(
     const A* __restrict__ zxg, int64_t row_stride, float* __restrict__ state, const int32_t* __restrict__ qo_indptr,
     const int64_t* __restrict__ pos0, const int32_t* __restrict__ state_slot, A* __restrict__ out, int width) {
-    __shared__ float agg_a[4][64], agg_b[4][64];
+    __shared__ float agg_a[GRU_NSEG][GRU_CB], agg_b[GRU_NSEG][GRU_CB];
     const int b = blockIdx.y;
     const int slot = state_slot[b];
     if (slot < 0) return;
     const int64_t q0 = qo_indptr ? qo_indptr[b] : b;
     const int64_t n = qo_indptr ? qo_indptr[b + 1] - q0 : 1;
     if (n <= 0) return;
-    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-    const int c = blockIdx.x * 64 + lane;
-    const bool live = c < width;
-    float carry = (live && pos0[b] > 0) ? state[(int64_t)slot * width + c] : 0.f;
-    for (int64_t base = 0; base < n; base += SEG * 4) {
-        const int64_t t0 = base + (int64_t)wv * SEG;
-        float pa[SEG], ps[SEG], gg[SEG];
-        float a_run = 1.f, s_run = 0.f;
+    const int seg = threadIdx.x >> 4, cl = (threadIdx.x & 15) * 2;
+    const int c = blockIdx.x * GRU_CB + cl;
+    const bool live0 = c < width, live1 = c + 1 < width;
+    const bool had = pos0[b] > 0;
+    float carry0 = (live0 && had) ? state[(int64_t)slot * width + c] : 0.f;
+    float carry1 = (live1 && had) ? state[(int64_t)slot * width + c + 1] : 0.f;
+    for (int64_t base = 0; base < n; base += SEG * GRU_NSEG) {
+        const int64_t t0 = base + (int64_t)seg * SEG;
+        float pa0[SEG], ps0[SEG], gg0[SEG], pa1[SEG], ps1[SEG], gg1[SEG];
+        float a0 = 1.f, s0 = 0.f, a1 = 1.f, s1 = 0.f;
 #pragma unroll
         for (int i = 0; i < SEG; ++i) {
             const int64_t t = t0 + i;
-            if (live && t < n) {
+            gg0[i] = gg1[i] = 0.f;
+            if (t < n) {
                 const A* r = zxg + (q0 + t) * row_stride;
-                const float z = sigmoidf_(ldf(r, c));
-                const float u = ldf(r, (int64_t)width + c);
-                const float cand = u >= 0.f ? u + 0.5f : sigmoidf_(u);
-                const float g = ldf(r, 2 * (int64_t)width + c);
-                gg[i] = g * sigmoidf_(g);
-                s_run = (1.0f - z) * s_run + z * cand;
-                a_run *= (1.0f - z);
-            } else gg[i] = 0.f;
-            pa[i] = a_run;
-            ps[i] = s_run;
+                if (live0) {
+                    const float z = sigm<A>(ldf(r, c));
+                    const float u = ldf(r, (int64_t)width + c);
+                    const float cand = u >= 0.f ? u + 0.5f : sigm<A>(u);
+                    const float g = ldf(r, 2 * (int64_t)width + c);
+                    gg0[i] = g * sigm<A>(g);
+                    s0 = (1.0f - z) * s0 + z * cand;
+                    a0 *= (1.0f - z);
+                }
+                if (live1) {
+                    const float z = sigm<A>(ldf(r, c + 1));
+                    const float u = ldf(r, (int64_t)width + c + 1);
+                    const float cand = u >= 0.f ? u + 0.5f : sigm<A>(u);
+                    const float g = ldf(r, 2 * (int64_t)width + c + 1);
+                    gg1[i] = g * sigm<A>(g);
+                    s1 = (1.0f - z) * s1 + z * cand;
+                    a1 *= (1.0f - z);
+                }
+            }
+            pa0[i] = a0; ps0[i] = s0; pa1[i] = a1; ps1[i] = s1;
         }
         __syncthreads();                   // the previous round's readers are done
-        agg_a[wv][lane] = a_run;
-        agg_b[wv][lane] = s_run;
+        agg_a[seg][cl] = a0; agg_b[seg][cl] = s0;
+        agg_a[seg][cl + 1] = a1; agg_b[seg][cl + 1] = s1;
         __syncthreads();
-        float in = carry;                  // state before this wave's first token
-        for (int k = 0; k < wv; ++k) in = agg_a[k][lane] * in + agg_b[k][lane];
-        float last = in;
-        for (int k = wv; k < 4; ++k) last = agg_a[k][lane] * last + agg_b[k][lane];
-        carry = last;                      // state after the round's last token (segments past the end are identities)
+        float in0 = carry0, in1 = carry1;  // state before this thread's first token
+        for (int k = 0; k < seg; ++k) {
+            in0 = agg_a[k][cl] * in0 + agg_b[k][cl];
+            in1 = agg_a[k][cl + 1] * in1 + agg_b[k][cl + 1];
+        }
+        float l0 = in0, l1 = in1;
+        for (int k = seg; k < GRU_NSEG; ++k) {
+            l0 = agg_a[k][cl] * l0 + agg_b[k][cl];
+            l1 = agg_a[k][cl + 1] * l1 + agg_b[k][cl + 1];
+        }
+        carry0 = l0;                       // state after the round's last token (segments past the end are identities)
+        carry1 = l1;
 #pragma unroll
         for (int i = 0; i < SEG; ++i) {
             const int64_t t = t0 + i;
-            if (live && t < n) stf(out, (q0 + t) * (int64_t)width + c, (pa[i] * in + ps[i]) * gg[i]);
+            if (t < n) {
+                if (live0) stf(out, (q0 + t) * (int64_t)width + c, (pa0[i] * in0 + ps0[i]) * gg0[i]);
+                if (live1) stf(out, (q0 + t) * (int64_t)width + c + 1, (pa1[i] * in1 + ps1[i]) * gg1[i]);
+            }
         }
     }
-    if (live && wv == 0) state[(int64_t)slot * width + c] = carry;
+    if (seg == 0) {
+        if (live0) state[(int64_t)slot * width + c] = carry0;
+        if (live1) state[(int64_t)slot * width + c + 1] = carry1;
+    }
 }
 
 // one token per sequence (a decode step): thread = (sequence, channel)
@@ -207,14 +332,14 @@ __global__ __launch_bounds__(256) void mingru_step_kernel(
         const int slot = state_slot[b];
         if (slot < 0) { stf(out, id, 0.f); continue; }
         const A* r = zxg + b * row_stride;
-        const float z = sigmoidf_(ldf(r, c));
+        const float z = sigm<A>(ldf(r, c));
         const float u = ldf(r, (int64_t)width + c);
-        const float cand = u >= 0.f ? u + 0.5f : sigmoidf_(u);
+        const float cand = u >= 0.f ? u + 0.5f : sigm<A>(u);
         const float g = ldf(r, 2 * (int64_t)width + c);
         float* sp = state + (int64_t)slot * width + c;
         const float s = (1.0f - z) * (pos0[b] > 0 ? *sp : 0.f) + z * cand;
         *sp = s;
-        stf(out, id, s * (g * sigmoidf_(g)));
+        stf(out, id, s * (g * sigm<A>(g)));
     }
 }
 
@@ -222,18 +347,35 @@ template <typename A>
 static void launch_boundary(const void* m, int64_t m_stride, const float* res, const float* w_post, float* hist, int64_t hist_stride,
                             int hist_slot, int n_mix, const float* mix, float* x_out, const float* w_pre, float* y_f32, void* y_act,
                             int64_t n_tok, int width, float eps, hipStream_t s) {
-    hipLaunchKernelGGL(boundary_norm_kernel<A>, dim3((unsigned)n_tok), dim3(256), 0, s, (const A*)m, m_stride, res, w_post, hist,
-                       hist_stride, hist_slot, n_mix, mix, x_out, w_pre, y_f32, (A*)y_act, width, eps);
+    const bool vec = width % 4 == 0 && m_stride % 4 == 0 && hist_stride % 4 == 0 && nvx_aligned16(m) && nvx_aligned16(res) &&
+                     nvx_aligned16(w_post) && nvx_aligned16(hist) && nvx_aligned16(x_out) && nvx_aligned16(w_pre) && nvx_aligned16(y_f32) &&
+                     nvx_aligned16(y_act);
+#define NVX_BOUNDARY_REG(VPT)                                                                                                         \
+    hipLaunchKernelGGL((boundary_norm_reg_kernel<A, VPT>), dim3((unsigned)n_tok), dim3(256), 0, s, (const A*)m, m_stride, res, w_post, \
+                       hist, hist_stride, hist_slot, n_mix, mix, x_out, w_pre, y_f32, (A*)y_act, width, eps)
+    if (vec && width <= 1024) NVX_BOUNDARY_REG(1);
+    else if (vec && width <= 2048) NVX_BOUNDARY_REG(2);
+    else if (vec && width <= 4096) NVX_BOUNDARY_REG(4);
+    else if (vec && width <= 8192) NVX_BOUNDARY_REG(8);
+    else
+        hipLaunchKernelGGL(boundary_norm_kernel<A>, dim3((unsigned)n_tok), dim3(256), 0, s, (const A*)m, m_stride, res, w_post, hist,
+                           hist_stride, hist_slot, n_mix, mix, x_out, w_pre, y_f32, (A*)y_act, width, eps);
+#undef NVX_BOUNDARY_REG
 }
 
 template <typename A>
 static void launch_canon(const float* h, const float* taps, int taps_n, float* state, const int32_t* tok_seq, const int32_t* qo_indptr,
                          const int64_t* pos0, const int32_t* state_slot, void* out, int64_t n_tok, int64_t n_seq, int width,
                          hipStream_t s) {
-    int64_t blocks = (n_tok * width + 255) / 256;
-    if (blocks > 256 * 64) blocks = 256 * 64;
-    hipLaunchKernelGGL(canon_conv_kernel<A>, dim3((unsigned)blocks), dim3(256), 0, s, h, taps, taps_n, (const float*)state, tok_seq,
-                       qo_indptr, pos0, state_slot, (A*)out, n_tok, width);
+    if (width % 4 == 0 && n_tok <= 65535 && nvx_aligned16(h) && nvx_aligned16(state) && nvx_aligned16(out)) {
+        hipLaunchKernelGGL(canon_conv_vec_kernel<A>, dim3((unsigned)((width / 4 + 255) / 256), (unsigned)n_tok), dim3(256), 0, s, h, taps,
+                           taps_n, (const float*)state, tok_seq, qo_indptr, pos0, state_slot, (A*)out, width);
+    } else {
+        int64_t blocks = (n_tok * width + 255) / 256;
+        if (blocks > 256 * 64) blocks = 256 * 64;
+        hipLaunchKernelGGL(canon_conv_kernel<A>, dim3((unsigned)blocks), dim3(256), 0, s, h, taps, taps_n, (const float*)state, tok_seq,
+                           qo_indptr, pos0, state_slot, (A*)out, n_tok, width);
+    }
     if (taps_n > 1)
         hipLaunchKernelGGL(canon_state_kernel, dim3((unsigned)((width + 255) / 256), (unsigned)n_seq), dim3(256), 0, s, h, taps_n, state,
                            qo_indptr, pos0, state_slot, width);
@@ -249,7 +391,7 @@ static void launch_mingru(const void* zxg, int64_t row_stride, float* state, con
                            state_slot, (A*)out, n_seq, width);
         return;
     }
-    hipLaunchKernelGGL((mingru_scan_kernel<A, 8>), dim3((unsigned)((width + 63) / 64), (unsigned)n_seq), dim3(256), 0, s, (const A*)zxg,
+    hipLaunchKernelGGL((mingru_scan_kernel<A, 8>), dim3((unsigned)((width + GRU_CB - 1) / GRU_CB), (unsigned)n_seq), dim3(256), 0, s, (const A*)zxg,
                        row_stride, state, qo_indptr, pos0, state_slot, (A*)out, width);
 }
 

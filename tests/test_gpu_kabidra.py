@@ -161,17 +161,17 @@ def test_canon_conv_continues_over_cuts_of_every_length(taps):
 
 @pytest.mark.parametrize("width", [24, 64, 130])
 def test_mingru_scan_over_cuts_and_round_borders(width):
-    """The scan works in rounds of 32 tokens: lengths around one and several rounds, steps of one token, a long memory
+    """The scan works in rounds of 128 tokens: lengths around one and several rounds, steps of one token, a long memory
     (update gates near zero) so that a lost or stale state shows."""
     from nano_vllm_x_amd import ops
     g = torch.Generator().manual_seed(width)
-    n_tok = {0: 131, 1: 33, 2: 64}
+    n_tok = {0: 300, 1: 129, 2: 128}
     pre = {i: (torch.randn(n, width, generator=g) - 3.0, 2 * torch.randn(n, width, generator=g), torch.randn(n, width, generator=g))
            for i, n in n_tok.items()}
     want = {i: ko.gru_scan(*p)[0] for i, p in pre.items()}
     state = torch.full((4, width), 5.0).cuda()
     slot = {0: 3, 1: 1, 2: 0}
-    cuts = {0: [31, 1, 1, 32, 2, 64], 1: [32, 1], 2: [64]}
+    cuts = {0: [127, 1, 1, 128, 2, 41], 1: [128, 1], 2: [128]}
     at = {i: 0 for i in pre}
     got = {i: [] for i in pre}
     while any(at[i] < n_tok[i] for i in pre):
@@ -224,6 +224,42 @@ def test_latent_attn_sees_exactly_the_causal_prefix(heads, rank):
                 want = (p[:, None] * c[:n]).sum(0) * gate[t, h]
                 assert torch.allclose(out[h, t].double(), want, atol=1e-4), (b, l, h)
             t += 1
+
+
+@pytest.mark.parametrize("fmt", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("heads,rank", [(1, 32), (3, 96), (16, 256), (20, 512), (5, 40)])
+def test_latent_attn_16_bit_formats_on_the_matrix_cores(fmt, heads, rank):
+    """Ranks that are multiples of 32 take the matrix-core kernel (one, several and a partly filled group of 16 heads; key
+    counts that are not multiples of its tile of 16 nor of its four waves), another rank the plain one.  Against float64
+    on the rounded inputs; peaked scores, scattered slots, one token per sequence (a decode step) and ragged steps."""
+    from nano_vllm_x_amd import ops
+    g = torch.Generator().manual_seed(rank + heads)
+    pool = torch.randn(1300, rank, generator=g).to(fmt)
+    perm = torch.randperm(1300, generator=g).to(torch.int32)
+    for kv_len, q_len in (([300, 517, 3], [44, 3, 3]), ([1, 70, 129], [1, 1, 1])):
+        idx, o = [], 0
+        for n in kv_len:
+            idx.append(perm[o:o + n])
+            o += n
+        t_all = sum(q_len)
+        q = (torch.randn(heads, t_all, rank, generator=g) * 0.5).to(fmt)
+        gate = torch.rand(t_all, heads, generator=g)
+        scale = 3.0 / rank ** 0.5
+        decode = all(n == 1 for n in q_len)
+        lay = _layout(ops, q_len, [a - b for a, b in zip(kv_len, q_len)], [0, 1, 2], decode)
+        starts = torch.tensor([0, kv_len[0], kv_len[0] + kv_len[1]], dtype=torch.int64)
+        out = ops.latent_attn(q.cuda(), pool.cuda(), torch.cat(idx).cuda(), starts.cuda(), torch.tensor(kv_len, dtype=torch.int32).cuda(),
+                              lay, scale, gate=gate.cuda()).float().cpu()
+        t = 0
+        for b in range(3):
+            c = pool[idx[b].long()].double()
+            for l in range(q_len[b]):
+                n = kv_len[b] - q_len[b] + l + 1
+                for h in range(heads):
+                    p = torch.softmax(scale * (c[:n] @ q[h, t].double()), 0)
+                    want = (p[:, None] * c[:n]).sum(0) * gate[t, h]
+                    assert torch.allclose(out[h, t].double(), want, atol=3e-2 if fmt == torch.bfloat16 else 4e-3, rtol=1e-2), (b, l, h)
+                t += 1
 
 
 # ---- the model through the engine ----------------------------------------------------------------------------------
