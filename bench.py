@@ -459,7 +459,7 @@ def _kernel_table(z, t_pre, n_dec, ctx):
         resb = res.to(bf)
         add("qwen3 rmsnorm+residual", phase, _time_us(lambda: ops.rmsnorm(m, wv.to(bf), 1e-5, resb)), bytes_=t * w * 8)
         st = torch.zeros(n_seq + 1, 3, w, device=dev)
-        taps = torch.randn(w, 4, device=dev)
+        taps = torch.randn(4, w, device=dev)
         add("canon_conv", phase, _time_us(lambda: ops.canon_conv(res, taps, st, lay, bf)), bytes_=t * w * 6 + n_seq * 3 * w * 8, like="(none)")
         zxg = torch.randn(t, 3 * w, device=dev).to(bf)
         gs = torch.zeros(n_seq + 1, w, device=dev)

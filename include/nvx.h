@@ -458,7 +458,8 @@ int nvx_lmhead_sample_f16(const void* w_packed, int64_t n_rows, int64_t k, const
  *     hist[hist_slot][t] = r                                             (hist_slot >= 0; slots hist_stride floats apart)
  *     x = sum_{j < n_mix} mix[j] * hist[j][t]   (n_mix > 0; hist_slot < n_mix is r itself)   else x = r
  *     x_out[t] = x;   w_pre != NULL:  y = x / sqrt(mean(x^2) + eps) * (1 + w_pre)  ->  y_f32 or y_act (exactly one)
- * nvx_canon_conv:  out[t] = h[t] + sum_j taps[:, j] * h[t - (taps_n - 1) + j]  over the tokens of t's own sequence;
+ * nvx_canon_conv:  out[t] = h[t] + sum_j taps[j] * h[t - (taps_n - 1) + j]  over the tokens of t's own sequence (taps: taps_n
+ *     rows of `width`);
  *     inputs before this step come from state[slot] (taps_n - 1 rows of `width`, oldest first), which is then
  *     replaced by the sequence's last taps_n - 1 inputs.
  * nvx_relu2:  y = max(x, 0)^2, element by element.

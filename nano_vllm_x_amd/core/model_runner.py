@@ -174,6 +174,15 @@ class ModelRunner:
             self.kv_cache = SeqStateCache(self.dtype, self.device, kv_cache_size, self.state_slots, self.model.latent_ranks(),
                                           self.model.state_shapes())
             self.attn_backend = SeqStateBackend(self.kv_cache, self.device)
+            # decode steps as one hipGraph per batch size, as for paged attention: the device block table gives every
+            # running sequence a row of slot ids, and the state slot of each row of the step travels in a buffer of its own
+            self.block_table = BlockTable(self.max_bs, 2 * self.max_bs + 1, 2 * self.context_len, self.device)
+            self._state_slot_dev = torch.full((self.max_bs,), -1, dtype=torch.int32, device=self.device)
+            self._state_slot_hosts = [torch.full((self.max_bs,), -1, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+            self._state_slot_turn = 0
+            if not self.enforce_eager:
+                self.graph = HIPGraph()
+                self.capture_graph()
             return
         self.kv_cache = KVCachePool(dtype=self.dtype, device=self.device, num_tokens=kv_cache_size,
                                     num_layers=self.num_layers, num_heads=self.num_kv_heads, head_dim=self.head_dim,
@@ -399,9 +408,12 @@ class ModelRunner:
         # keep the device block table in step with what the scheduler decided: rows are (re)written from the
         # step's own slot lists, sequence by sequence, so a decode step that had to run outside the graph
         # (no free row, a list longer than a row) does not keep its batch off the graph path afterwards
-        if self.graph is not None and self.family == "paged_kv":
-            t = self.attn_backend.last_table
-            self.block_table.write_rows(batch.seqs, t["paged_kv_indices"], t["paged_kv_indptr"])
+        if self.graph is not None:
+            if self.family == "paged_kv":
+                t = self.attn_backend.last_table
+                self.block_table.write_rows(batch.seqs, t["paged_kv_indices"], t["paged_kv_indptr"])
+            else:
+                self.block_table.write_rows(batch.seqs, md.kv_indices, md.kv_indptr)
         return hidden
 
     def _run_stage(self, input_ids: torch.Tensor, positions: torch.Tensor) -> Optional[torch.Tensor]:
@@ -430,6 +442,12 @@ class ModelRunner:
         bs = batch.num_seqs
         padded = self.graph.match_bs(bs)
         self.block_table.stage_decode_step(batch.seqs, ids_on_device)
+        if self.family == "seq_state":
+            self._state_slot_turn ^= 1
+            host = self._state_slot_hosts[self._state_slot_turn]
+            host.fill_(-1)                    # rows past the batch are padding: no state is read or written for them
+            host[:bs] = torch.tensor([s.state_slot for s in batch.seqs], dtype=torch.int32)
+            self._state_slot_dev.copy_(host, non_blocking=True)
         self.graph.replay(padded)
         return self.graph.get_output_buffer("hidden_states")[:bs]
 
@@ -438,6 +456,14 @@ class ModelRunner:
         bt = self.block_table
         torch.ops.nvx.decode_step_setup(bt.step_dev, bt.max_bs, bs, bt.table, bt.pad_start, bt.kv_start, bt.kv_len, bt.out_slots,
                                         bt.positions, bt.input_ids, self._sample_out)
+        if self.family == "seq_state":
+            from ..layers.seq_state import SeqStateMetadata
+            md = SeqStateMetadata(forward_mode=ForwardMode.DECODE, cache=self.kv_cache,
+                                  layout=ops.StepLayout(bs, bs, bt.positions[:bs], self._state_slot_dev[:bs]),
+                                  kv_indices=bt.table.view(-1), kv_start=bt.kv_start[:bs], kv_len=bt.kv_len[:bs],
+                                  out_slots=bt.out_slots[:bs], kv_indptr=None)
+            with attention_kv_cache(self.model, md):
+                return self.model(bt.input_ids[:bs], bt.positions[:bs])
         torch.ops.nvx.decode_plan(bt.kv_len[:bs], bt.kv_start[:bs], bt.out_slots[:bs], self.num_kv_heads, self.decode_ws.plan)
         wrapper = self._graph_wrappers[bs]
         md = AttentionMetadata(forward_mode=ForwardMode.DECODE, kv_cache=self.kv_cache, output_kv_indices=bt.out_slots[:bs],
@@ -470,9 +496,10 @@ class ModelRunner:
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
             for bs in reversed(sizes):
-                w = PagedDecodeWrapper(None, "NHD", use_cuda_graph=True)
-                w.bind_table(bt.table.view(-1), bt.kv_start, bt.kv_len, bs, self.decode_ws, qkv_fused=True)
-                self._graph_wrappers[bs] = w
+                if self.family == "paged_kv":
+                    w = PagedDecodeWrapper(None, "NHD", use_cuda_graph=True)
+                    w.bind_table(bt.table.view(-1), bt.kv_start, bt.kv_len, bs, self.decode_ws, qkv_fused=True)
+                    self._graph_wrappers[bs] = w
                 self._decode_forward(bs)   # warm-up outside capture (library handles, allocator pool)
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()

@@ -131,7 +131,7 @@ __global__ __launch_bounds__(256) void boundary_norm_reg_kernel(
 }
 
 // ---- canon: h + causal convolution over time, per channel -----------------------------------------------------------
-// taps[c][j] multiplies the input (taps_n - 1 - j) tokens back.  state[slot][r] (r < taps_n - 1) is the input at position
+// taps[j][c] (taps_n rows of `width`) multiplies channel c of the input (taps_n - 1 - j) tokens back.  state[slot][r] (r < taps_n - 1) is the input at position
 // pos0 - (taps_n - 1) + r.
 template <typename A>
 __global__ __launch_bounds__(256) void canon_conv_kernel(
@@ -155,7 +155,7 @@ __global__ __launch_bounds__(256) void canon_conv_kernel(
             float v;
             if (s >= 0) v = h[(q0 + s) * width + c];
             else v = has_state ? state[((int64_t)slot * hist_n + (hist_n + s)) * width + c] : 0.f;
-            acc += taps[(int64_t)c * taps_n + j] * v;
+            acc += taps[(int64_t)j * width + c] * v;
         }
         stf(out, id, acc);
     }
@@ -184,8 +184,7 @@ __global__ __launch_bounds__(256) void canon_conv_vec_kernel(
         if (s >= 0) v = *reinterpret_cast<const f32x4v*>(h + (q0 + s) * width + c);
         else if (has_state) v = *reinterpret_cast<const f32x4v*>(state + ((int64_t)slot * hist_n + (hist_n + s)) * width + c);
         else continue;
-        const float* tp = taps + (int64_t)c * taps_n + j;
-        acc += f32x4v{tp[0], tp[taps_n], tp[2 * taps_n], tp[3 * taps_n]} * v;
+        acc += *reinterpret_cast<const f32x4v*>(taps + (int64_t)j * width + c) * v;
     }
     st4(out + t * width + c, acc);
 }
@@ -232,7 +231,7 @@ __device__ __forceinline__ float sigmoidf_(float v) { return 1.0f / (1.0f + expf
 // 16-bit activation formats: the hardware exponential (relative error ~1e-6, far below the format's own rounding)
 template <typename A> __device__ __forceinline__ float sigm(float v) {
     if constexpr (sizeof(A) == 4) return 1.0f / (1.0f + expf(-v));
-    else return 1.0f / (1.0f + __expf(-v));
+    else return __builtin_amdgcn_rcpf(1.0f + __expf(-v));
 }
 
 // A workgroup takes GRU_CB channels of one sequence and walks its tokens in rounds of GRU_NSEG * SEG tokens: thread
@@ -256,6 +255,8 @@ __global__ __launch_bounds__(256) void mingru_scan_kernel(
     const int c = blockIdx.x * GRU_CB + cl;
     const bool live0 = c < width, live1 = c + 1 < width;
     const bool had = pos0[b] > 0;
+    // the pair can be moved as one value when both channels exist and every row keeps the pair's alignment
+    const bool pair_ok = live1 && width % 2 == 0 && row_stride % 2 == 0 && (reinterpret_cast<uintptr_t>(zxg) % (2 * sizeof(A))) == 0;
     float carry0 = (live0 && had) ? state[(int64_t)slot * width + c] : 0.f;
     float carry1 = (live1 && had) ? state[(int64_t)slot * width + c + 1] : 0.f;
     for (int64_t base = 0; base < n; base += SEG * GRU_NSEG) {
@@ -268,21 +269,28 @@ __global__ __launch_bounds__(256) void mingru_scan_kernel(
             gg0[i] = gg1[i] = 0.f;
             if (t < n) {
                 const A* r = zxg + (q0 + t) * row_stride;
-                if (live0) {
-                    const float z = sigm<A>(ldf(r, c));
-                    const float u = ldf(r, (int64_t)width + c);
-                    const float cand = u >= 0.f ? u + 0.5f : sigm<A>(u);
-                    const float g = ldf(r, 2 * (int64_t)width + c);
-                    gg0[i] = g * sigm<A>(g);
+                float zz[2], uu[2], gq[2];
+                if (pair_ok) {             // both channels with one load each (the pair is aligned to its own size)
+                    typedef A a2 __attribute__((ext_vector_type(2)));
+                    const a2 zv = *reinterpret_cast<const a2*>(r + c), uv = *reinterpret_cast<const a2*>(r + width + c),
+                             gv = *reinterpret_cast<const a2*>(r + 2 * (int64_t)width + c);
+                    zz[0] = (float)zv.x; zz[1] = (float)zv.y; uu[0] = (float)uv.x; uu[1] = (float)uv.y; gq[0] = (float)gv.x; gq[1] = (float)gv.y;
+                } else {
+                    zz[0] = live0 ? ldf(r, c) : 0.f; uu[0] = live0 ? ldf(r, (int64_t)width + c) : 0.f; gq[0] = live0 ? ldf(r, 2 * (int64_t)width + c) : 0.f;
+                    zz[1] = live1 ? ldf(r, c + 1) : 0.f; uu[1] = live1 ? ldf(r, (int64_t)width + c + 1) : 0.f;
+                    gq[1] = live1 ? ldf(r, 2 * (int64_t)width + c + 1) : 0.f;
+                }
+                {
+                    const float z = sigm<A>(zz[0]);
+                    const float cand = uu[0] >= 0.f ? uu[0] + 0.5f : sigm<A>(uu[0]);
+                    gg0[i] = gq[0] * sigm<A>(gq[0]);
                     s0 = (1.0f - z) * s0 + z * cand;
                     a0 *= (1.0f - z);
                 }
-                if (live1) {
-                    const float z = sigm<A>(ldf(r, c + 1));
-                    const float u = ldf(r, (int64_t)width + c + 1);
-                    const float cand = u >= 0.f ? u + 0.5f : sigm<A>(u);
-                    const float g = ldf(r, 2 * (int64_t)width + c + 1);
-                    gg1[i] = g * sigm<A>(g);
+                {
+                    const float z = sigm<A>(zz[1]);
+                    const float cand = uu[1] >= 0.f ? uu[1] + 0.5f : sigm<A>(uu[1]);
+                    gg1[i] = gq[1] * sigm<A>(gq[1]);
                     s1 = (1.0f - z) * s1 + z * cand;
                     a1 *= (1.0f - z);
                 }
@@ -367,7 +375,7 @@ template <typename A>
 static void launch_canon(const float* h, const float* taps, int taps_n, float* state, const int32_t* tok_seq, const int32_t* qo_indptr,
                          const int64_t* pos0, const int32_t* state_slot, void* out, int64_t n_tok, int64_t n_seq, int width,
                          hipStream_t s) {
-    if (width % 4 == 0 && n_tok <= 65535 && nvx_aligned16(h) && nvx_aligned16(state) && nvx_aligned16(out)) {
+    if (width % 4 == 0 && n_tok <= 65535 && nvx_aligned16(h) && nvx_aligned16(state) && nvx_aligned16(out) && nvx_aligned16(taps)) {
         hipLaunchKernelGGL(canon_conv_vec_kernel<A>, dim3((unsigned)((width / 4 + 255) / 256), (unsigned)n_tok), dim3(256), 0, s, h, taps,
                            taps_n, (const float*)state, tok_seq, qo_indptr, pos0, state_slot, (A*)out, width);
     } else {

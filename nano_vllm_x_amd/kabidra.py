@@ -101,9 +101,10 @@ class KabidraLayer(nn.Module):
             self.mixer = LatentAttention(w, m["heads"], m["dim"], m["vdim"], m["q_rank"], m["kv_rank"], m["scale"], cfg.eps, layer_id=i)
         self.mlp = SquaredReLUMLP(w, spec["mlp"]["ff"]) if spec["mlp"] is not None else None
         # norm weights are stored as deviations from one; norms, taps and depth weights stay float32 in every format
-        self.norm1, self.norm1b, self.canon1 = _f32(w), _f32(w), _f32(w, cfg.taps)
+        # (the taps are kept as (taps, width): a tap's weights for neighbouring channels are neighbours in memory)
+        self.norm1, self.norm1b, self.canon1 = _f32(w), _f32(w), _f32(cfg.taps, w)
         if self.mlp is not None:
-            self.norm2, self.norm2b, self.canon2 = _f32(w), _f32(w), _f32(w, cfg.taps)
+            self.norm2, self.norm2b, self.canon2 = _f32(w), _f32(w), _f32(cfg.taps, w)
         self.dwa = _f32(i + 2)
 
 
@@ -204,7 +205,10 @@ class KabidraForCausalLM(nn.Module):
         if not (head[:1] == "l" and head[1:].isdigit() and int(head[1:]) < len(self.layers)):
             raise KeyError(f"unexpected tensor {name!r}")
         layer = self.layers[int(head[1:])]
-        if rest in ("norm1", "norm1b", "norm2", "norm2b", "canon1", "canon2", "dwa") and hasattr(layer, rest):
+        if rest in ("canon1", "canon2") and hasattr(layer, rest):
+            w = w.t()                        # stored (width, taps), kept (taps, width)
+            return put(getattr(layer, rest))
+        if rest in ("norm1", "norm1b", "norm2", "norm2b", "dwa") and hasattr(layer, rest):
             return put(getattr(layer, rest))
         if rest == "mlp.up" and layer.mlp is not None:
             return put(layer.mlp.up_proj.weight)

@@ -42,6 +42,7 @@ class SeqStateMetadata:
     kv_start: torch.Tensor          # int64 (B): where each sequence's list starts in kv_indices
     kv_len: torch.Tensor            # int32 (B): tokens of each sequence, this step's included
     out_slots: torch.Tensor         # int64 (T): slot of every token computed in this step
+    kv_indptr: Optional[torch.Tensor] = None     # int32 (B+1): kv_start with the total appended (steps built from a batch)
 
 
 class SeqStateBackend:
@@ -75,5 +76,8 @@ class SeqStateBackend:
             np.cumsum(q_lens, out=qo[1:])
             tok_seq = np.repeat(np.arange(n, dtype=np.int32), q_lens)
             layout = ops.StepLayout(t, n, self._up(pos0), self._up(slot), self._up(qo), self._up(tok_seq))
+        kv_indptr = np.zeros(n + 1, dtype=np.int32)
+        np.cumsum(kv_lens, out=kv_indptr[1:])
         return SeqStateMetadata(forward_mode=batch.forward_mode, cache=self.cache, layout=layout, kv_indices=self._up(flat),
-                                kv_start=self._up(kv_start), kv_len=self._up(kv_lens), out_slots=self._up(out_slots))
+                                kv_start=self._up(kv_start), kv_len=self._up(kv_lens), out_slots=self._up(out_slots),
+                                kv_indptr=self._up(kv_indptr))

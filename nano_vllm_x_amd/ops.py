@@ -747,15 +747,16 @@ def boundary_norm(m, w_post, eps: float, res=None, hist=None, hist_slot: int = -
 
 
 def canon_conv(h, taps, state, layout: StepLayout, dtype):
-    """h + causal convolution over time per channel.  h (T, width) float32; taps (width, taps_n) float32; state
+    """h + causal convolution over time per channel.  h (T, width) float32; taps (taps_n, width) float32, row j multiplying
+    the input taps_n - 1 - j tokens back; state
     (slots, taps_n - 1, width) float32, read for the inputs before this step and replaced by each sequence's last ones.
     Returns (T, width) in `dtype`."""
     _dev(h, taps, state)
     _f32c(h, "canon_conv: h")
     _f32c(taps, "canon_conv: taps")
     t, width = h.shape
-    taps_n = taps.shape[1]
-    _need(t == layout.n_tok and taps.shape[0] == width, "canon_conv: shapes")
+    taps_n = taps.shape[0]
+    _need(t == layout.n_tok and taps.dim() == 2 and taps.shape[1] == width, "canon_conv: shapes")
     n_slots = 0
     if taps_n > 1:
         _f32c(state, "canon_conv: state")

@@ -145,7 +145,7 @@ def test_canon_conv_continues_over_cuts_of_every_length(taps):
         lens = [min(cuts[i].pop(0), len(full[i]) - at[i]) for i in live]
         h = torch.cat([full[i][at[i]:at[i] + n] for i, n in zip(live, lens)])
         decode = all(n == 1 for n in lens)
-        out = ops.canon_conv(h.cuda(), k.cuda(), state, _layout(ops, lens, [at[i] for i in live], [slot[i] for i in live], decode),
+        out = ops.canon_conv(h.cuda(), k.t().contiguous().cuda(), state, _layout(ops, lens, [at[i] for i in live], [slot[i] for i in live], decode),
                              torch.float32).cpu()
         o = 0
         for i, n in zip(live, lens):
@@ -155,7 +155,7 @@ def test_canon_conv_continues_over_cuts_of_every_length(taps):
     for i in full:
         assert torch.allclose(torch.cat(got[i]), want[i], atol=1e-5), f"sequence {i}"
     fresh = torch.randn(5, w, generator=g)
-    out = ops.canon_conv(fresh.cuda(), k.cuda(), state, _layout(ops, [5], [0], [2]), torch.float32).cpu()
+    out = ops.canon_conv(fresh.cuda(), k.t().contiguous().cuda(), state, _layout(ops, [5], [0], [2]), torch.float32).cpu()
     assert torch.allclose(out, ko.canon(fresh, k), atol=1e-5), "a sequence at position 0 must not read the slot's old tail"
 
 
@@ -411,6 +411,41 @@ def test_greedy_generation_through_the_engine(tmp_path, chunked):
         assert out[i] == oracle_greedy(w, cfg, p, new[i]), i
     assert eng.scheduler.state_slots.num_free() == 3
     eng.shutdown()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_steps_replay_a_captured_graph(tmp_path, dtype):
+    """With graphs on, every decode step replays the graph of its batch size, with prefill steps of later requests (eager
+    work on the same cache and state) between the replays; batch sizes change as requests end.  float32: the tokens are
+    the restatement's; bfloat16: the graph's tokens are those of eager steps (same kernels, same order)."""
+    from nano_vllm_x_amd.core.common import SamplingParams
+    from nano_vllm_x_amd.core.engine import Engine
+    cfg = make_cfg([GRU, ATT, GRU, ATT])
+    path = model_dir(tmp_path, cfg)
+    prompts = {f"r{k}": tokens(n, cfg["vocab"], 40 + k) for k, n in enumerate([9, 30, 2, 17, 5])}
+    new = {"r0": 25, "r1": 5, "r2": 12, "r3": 3, "r4": 8}
+
+    def run(eager):
+        eng = Engine(model=path, gpu_memory_utilization=0.5, max_bs=3, enforce_eager=eager, context_len=128, kv_cache_size=300,
+                     dtype=dtype, seed=5)
+        for i, p in prompts.items():
+            eng.add_sequence(i, list(p), SamplingParams(temperature=0.0, ignore_eos=True, max_new_tokens=new[i]))
+        out = {i: [] for i in prompts}
+        while eng.has_unfinished_sequences():
+            for o in eng.step():
+                out[o.seq_id].append(o.new_token_id)
+        stats = dict(eng.model_runner.stats)
+        eng.shutdown()
+        return out, stats
+
+    got, stats = run(False)
+    assert stats["graph_steps"] > 20 and stats["eager_decode_steps"] == 0
+    if dtype == "float32":
+        w = weights_of(cfg, 5)
+        for i, p in prompts.items():
+            assert got[i] == oracle_greedy(w, cfg, p, new[i]), i
+    else:
+        assert got == run(True)[0]
 
 
 def test_generate_entry_point(tmp_path):
