@@ -476,11 +476,24 @@ def _kernel_table(z, t_pre, n_dec, ctx):
         kvl = torch.full((n_seq,), kv_len, dtype=torch.int32, device=dev)
         q = torch.randn(h, t, r, device=dev).to(bf)
         us = _time_us(lambda: ops.latent_attn(q, pool, idx, kv_start, kvl, lay, 0.1), reps=3 if phase == "prefill" else 20)
+        # ... beside paged attention with 8 K/V heads of 128 over the same tokens
+        kc = torch.randn(n_seq * kv_len, 8, 128, device=dev).to(bf)
+        vc = torch.randn(n_seq * kv_len, 8, 128, device=dev).to(bf)
+        q128 = torch.randn(t, h * 128, device=dev).to(bf)
         if phase == "prefill":
             pairs = n_seq * q_len * (q_len + 1) // 2
             add("latent_attn", phase, us, flops=4.0 * h * r * pairs, like="paged_prefill")
+            plan = ops.prefill_plan_ws(n_seq, dev)
+            kv_indptr = torch.arange(0, n_seq + 1, dtype=torch.int32, device=dev) * kv_len
+            ops.prefill_plan(lay.qo_indptr, plan)
+            us = _time_us(lambda: ops.paged_prefill(q128, kc, vc, lay.qo_indptr, kv_indptr, idx, plan, h, 8, 0.1), reps=5)
+            add("qwen3 paged_prefill", phase, us, flops=4.0 * h * 128 * pairs)
         else:
             add("latent_attn", phase, us, bytes_=n_seq * kv_len * r * 2 + 2 * t * h * r * 2, like="paged_decode")
+            ws = ops.DecodeWorkspace(n_seq, h, 8, dev)
+            ops.decode_plan(kvl, kv_start, ws)
+            us = _time_us(lambda: ops.paged_decode(q128, kc, vc, idx, n_seq, ws, 0.1))
+            add("qwen3 paged_decode", phase, us, bytes_=n_seq * kv_len * 8 * 128 * 2 * 2 + 2 * t * h * 128 * 2)
     return rows
 
 

@@ -159,7 +159,7 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(
     }
 }
 
-// ---- the same on the matrix cores (16-bit formats, rank a multiple of 32, at most 512) -----------------------------------
+// ---- the same on the matrix cores (16-bit formats; rank 32 .. 256 in steps of 32, 320, 384, 448 or 512) -----------------------------------
 // One workgroup per (query token, group of 16 heads); its four waves take every fourth tile of 16 keys and merge at the
 // end.  Per tile:
 //   S^T (16 keys x 16 heads) = C_tile (16 x rank) . Q~^T (rank x 16)        v_mfma_f32_16x16x32, rank / 32 of them; the A
@@ -198,14 +198,15 @@ template <typename A> __device__ __forceinline__ float la_round(float v) { retur
 
 #define LA_PAD 8     // elements between the rows of a parked tile: 16-byte rows, and the four quarters hit different banks
 
-template <typename A, int RKM>      // RKM: k-steps of 32 the registers are sized for (rank <= 32 * RKM)
+template <typename A, int RKM>      // RKM = rank / 32, the k-steps of a score product (compile time: the loops below unroll into
+                                    // straight-line code, so the LDS reads of a tile run ahead of the products that use them)
 __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
     const A* __restrict__ q, const A* __restrict__ cache, const int32_t* __restrict__ kv_indices, const int64_t* __restrict__ kv_start,
     const int32_t* __restrict__ kv_len, const int32_t* __restrict__ qo_indptr, const int32_t* __restrict__ tok_seq,
     const float* __restrict__ gate, A* __restrict__ out, int heads, int rank, int64_t n_tok, float scale) {
     extern __shared__ float lds[];
     constexpr int NB2 = RKM;                   // pairs of 16-column blocks = rank / 32
-    const int steps = rank >> 5;
+    constexpr int steps = RKM;
     const int64_t t = blockIdx.x;
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, l16 = lane & 15, quarter = lane >> 4;
     const int head = blockIdx.y * 16 + l16;
@@ -221,7 +222,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
 #pragma unroll
     for (int ks = 0; ks < RKM; ++ks) {
         qb[ks] = nvx_u32x4{0u, 0u, 0u, 0u};
-        if (ks < steps && head < heads)
+        if (head < heads)
             qb[ks] = *reinterpret_cast<const nvx_u32x4*>(q + ((int64_t)head * n_tok + t) * rank + 32 * ks + 8 * quarter);
     }
     nvx_f32x4 o_acc[2 * NB2];
@@ -230,21 +231,37 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
     float m_run = -INFINITY, l_run = 0.f;      // of head l16; l_run: this quarter's keys only
 
     const int64_t n_tiles = (n_keys + 15) >> 4;
-    for (int64_t j = wv; j < n_tiles; j += 4) {
+    // A tile's rows hang on its slot ids, which hang on the table: two memory round trips in a row.  The ids are read two
+    // tiles ahead and the rows one tile ahead, so that neither wait stands in front of a tile's products.
+    nvx_u32x4 a_nxt[RKM];
+    auto slot_of = [&](int64_t j) {
         const int64_t key = j * 16 + l16;
-        const int slot = idx[key < n_keys ? key : 0];            // a key past the end reads a real row and is masked below
+        return idx[key < n_keys ? key : 0];                      // a key past the end reads a real row and is masked below
+    };
+    auto fetch = [&](int slot) {
         const A* row = cache + (int64_t)slot * rank;
+#pragma unroll
+        for (int ks = 0; ks < RKM; ++ks)
+            a_nxt[ks] = *reinterpret_cast<const nvx_u32x4*>(row + 32 * ks + 8 * quarter);
+    };
+    int slot_nxt = 0;
+    if (wv < n_tiles) fetch(slot_of(wv));
+    if (wv + 4 < n_tiles) slot_nxt = slot_of(wv + 4);
+    for (int64_t j = wv; j < n_tiles; j += 4) {
+        nvx_u32x4 a_cur[RKM];
+#pragma unroll
+        for (int ks = 0; ks < RKM; ++ks) a_cur[ks] = a_nxt[ks];
+        if (j + 4 < n_tiles) fetch(slot_nxt);
+        if (j + 8 < n_tiles) slot_nxt = slot_of(j + 8);
         nvx_f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ks = 0; ks < RKM; ++ks) {
-            if (ks < steps) {
-                const nvx_u32x4 a = *reinterpret_cast<const nvx_u32x4*>(row + 32 * ks + 8 * quarter);
-                *reinterpret_cast<nvx_u32x4*>(tile + l16 * row_elems + 32 * ks + 8 * quarter) = a;
-                sacc = la_mfma32<A>(a, qb[ks], sacc);
-            }
+            *reinterpret_cast<nvx_u32x4*>(tile + l16 * row_elems + 32 * ks + 8 * quarter) = a_cur[ks];
+            sacc = la_mfma32<A>(a_cur[ks], qb[ks], sacc);
         }
-        // the tile is parked before any lane reads it back transposed (one wave: its LDS operations complete in order)
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        // the tile is parked before any lane reads it back transposed (one wave: its LDS operations complete in order);
+        // the barrier is for the compiler, which must not move the reads below above the writes
+        asm volatile("" ::: "memory");
         float sv[4], mx = -INFINITY;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -255,6 +272,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
         mx = fmaxf(mx, xor32(mx));
         const float m_new = fmaxf(m_run, mx);                    // finite: a tile has at least one visible key
         const float alpha = __expf(m_run - m_new);
+        const bool rescale = __any(alpha != 1.0f);               // once the maxima have settled, most tiles change none
         m_run = m_new;
         l_run *= alpha;
         float p[4], ph[4];
@@ -269,34 +287,35 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
         const uint32_t* tile32 = reinterpret_cast<const uint32_t*>(tile);
 #pragma unroll
         for (int b2 = 0; b2 < NB2; ++b2) {
-            if (b2 < steps) {
+            {
                 uint32_t d[4];
 #pragma unroll
                 for (int r = 0; r < 4; ++r) d[r] = tile32[((4 * quarter + r) * row_elems + 32 * b2) / 2 + l16];
                 const uint2 even = make_uint2((d[0] & 0xffffu) | (d[1] << 16), (d[2] & 0xffffu) | (d[3] << 16));
                 const uint2 odd = make_uint2((d[0] >> 16) | (d[1] & 0xffff0000u), (d[2] >> 16) | (d[3] & 0xffff0000u));
-                o_acc[2 * b2] *= alpha;
-                o_acc[2 * b2 + 1] *= alpha;
+                if (rescale) {
+                    o_acc[2 * b2] *= alpha;
+                    o_acc[2 * b2 + 1] *= alpha;
+                }
                 o_acc[2 * b2] = la_mfma16<A>(even, p_hi, o_acc[2 * b2]);
                 o_acc[2 * b2] = la_mfma16<A>(even, p_lo, o_acc[2 * b2]);
                 o_acc[2 * b2 + 1] = la_mfma16<A>(odd, p_hi, o_acc[2 * b2 + 1]);
                 o_acc[2 * b2 + 1] = la_mfma16<A>(odd, p_lo, o_acc[2 * b2 + 1]);
             }
         }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");      // the reads are done before the next tile is parked
+        asm volatile("" ::: "memory");                          // (compiler) the reads stay above the next tile's writes
     }
 
     // merge the four waves' partial results: 2 and 3 into 0 and 1, then 1 into 0.  Every lane parks its own values; the lane
     // of the same number in the other wave holds the same head and columns.
-    const int vals = 8 * steps + 2;
+    constexpr int vals = 8 * steps + 2;
     auto park = [&](int region) {
         float* base = lds + (size_t)region * vals * 64 + lane;
 #pragma unroll
-        for (int i = 0; i < 2 * NB2; ++i)
-            if (i < 2 * steps) {
+        for (int i = 0; i < 2 * NB2; ++i) {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) base[(4 * i + r) * 64] = o_acc[i][r];
-            }
+            for (int r = 0; r < 4; ++r) base[(4 * i + r) * 64] = o_acc[i][r];
+        }
         base[(8 * steps) * 64] = m_run;
         base[(8 * steps + 1) * 64] = l_run;
     };
@@ -309,11 +328,10 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
         m_run = m_new;
         l_run = l_run * fa + l_o * fb;
 #pragma unroll
-        for (int i = 0; i < 2 * NB2; ++i)
-            if (i < 2 * steps) {
+        for (int i = 0; i < 2 * NB2; ++i) {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) o_acc[i][r] = o_acc[i][r] * fa + base[(4 * i + r) * 64] * fb;
-            }
+            for (int r = 0; r < 4; ++r) o_acc[i][r] = o_acc[i][r] * fa + base[(4 * i + r) * 64] * fb;
+        }
     };
     __syncthreads();                 // every wave is done with its tile: the memory changes hands
     if (wv >= 2) park(wv - 2);
@@ -331,7 +349,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
     A* orow = out + ((int64_t)head * n_tok + t) * rank;
 #pragma unroll
     for (int b2 = 0; b2 < NB2; ++b2) {
-        if (b2 < steps) {
+        {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {        // row i = 4 * quarter + r of the pair's blocks: columns 2 i (even) and 2 i + 1 (odd)
                 const int c = 32 * b2 + 2 * (4 * quarter + r);
@@ -353,17 +371,29 @@ static void launch_attn(const void* q, const void* cache, const int32_t* kv_indi
                         const int32_t* qo_indptr, const int32_t* tok_seq, const float* gate, void* out, int heads, int rank, int64_t n_tok,
                         float scale, hipStream_t s) {
     if constexpr (sizeof(A) == 2) {
-        if (rank % 32 == 0 && rank <= 512 && nvx_aligned16(q) && nvx_aligned16(cache) && nvx_aligned16(out) && n_tok <= 0x7fffffff) {
-            const int steps = rank / 32;
+        const int steps = rank / 32;
+        const bool built = steps <= 8 || steps == 10 || steps == 12 || steps == 14 || steps == 16;     // the ranks the kernel is built for
+        if (rank % 32 == 0 && built && nvx_aligned16(q) && nvx_aligned16(cache) && nvx_aligned16(out) && n_tok <= 0x7fffffff) {
             const size_t tiles = (size_t)4 * 16 * (rank + LA_PAD) * 2, merge = (size_t)2 * (8 * steps + 2) * 64 * 4;
             const size_t lds = tiles > merge ? tiles : merge;
             const dim3 grid((unsigned)n_tok, (unsigned)((heads + 15) / 16));
 #define NVX_LA_MFMA(RKM)                                                                                                            \
     hipLaunchKernelGGL((latent_attn_mfma_kernel<A, RKM>), grid, dim3(256), lds, s, (const A*)q, (const A*)cache, kv_indices, kv_start, \
                        kv_len, qo_indptr, tok_seq, gate, (A*)out, heads, rank, n_tok, scale)
-            if (steps <= 4) NVX_LA_MFMA(4);
-            else if (steps <= 8) NVX_LA_MFMA(8);
-            else NVX_LA_MFMA(16);
+            switch (steps) {
+                case 1: NVX_LA_MFMA(1); break;
+                case 2: NVX_LA_MFMA(2); break;
+                case 3: NVX_LA_MFMA(3); break;
+                case 4: NVX_LA_MFMA(4); break;
+                case 5: NVX_LA_MFMA(5); break;
+                case 6: NVX_LA_MFMA(6); break;
+                case 7: NVX_LA_MFMA(7); break;
+                case 8: NVX_LA_MFMA(8); break;
+                case 10: NVX_LA_MFMA(10); break;
+                case 12: NVX_LA_MFMA(12); break;
+                case 14: NVX_LA_MFMA(14); break;
+                default: NVX_LA_MFMA(16); break;
+            }
 #undef NVX_LA_MFMA
             return;
         }
