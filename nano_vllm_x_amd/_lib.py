@@ -13,6 +13,9 @@ import re
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # NVX_LIB_PATH: another build of the same library (A/B timing of two versions of a kernel in one job)
 LIB_PATH = os.environ.get("NVX_LIB_PATH") or os.path.join(_HERE, "libnvx_hip.so")
+# `make seq`: the entry points a seq-state model needs (its kernels, the sampler, the block table) and nothing else; loaded
+# only where the full library is absent
+SUBSET_LIB_PATH = os.path.join(_HERE, "libnvx_hip_seq.so")
 HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "nvx.h")
 
 
@@ -106,23 +109,48 @@ for _name in F16_ENTRY_POINTS:
     SIGNATURES[_name + "_f16"] = SIGNATURES[_name]
 
 
+class _SubsetLibrary:
+    """The subset library behind the same attribute access: an entry point it was not built with raises by name."""
+
+    def __init__(self, cdll, path):
+        self._cdll, self._path = cdll, path
+
+    def __getattr__(self, name):
+        try:
+            return getattr(self._cdll, name)
+        except AttributeError:
+            raise NvxLibraryError(f"{self._path} holds only the kernels of seq-state models and lacks {name}: build the full "
+                                  "library with `make -C nano_vllm_x_amd/csrc`") from None
+
+
+def is_subset() -> bool:
+    return isinstance(load(), _SubsetLibrary)
+
+
 def load():
-    """Load the HIP library once; raise loudly when it is absent (no fallback path exists)."""
+    """Load the HIP library once; raise loudly when it is absent (no fallback path exists).  Where only the subset library
+    of `make seq` has been built, that one is loaded: its entry points work, the others raise when called."""
     global _lib
     if _lib is not None:
         return _lib
-    if not os.path.exists(LIB_PATH):
+    subset = not os.path.exists(LIB_PATH) and not os.environ.get("NVX_LIB_PATH") and os.path.exists(SUBSET_LIB_PATH)
+    path = SUBSET_LIB_PATH if subset else LIB_PATH
+    if not os.path.exists(path):
         raise NvxLibraryError(
             f"{LIB_PATH} not found: build it with `make -C nano_vllm_x_amd/csrc` "
             "(or `python -c 'import __graft_entry__ as g; g.build()'`). There is no fallback path.")
-    lib = ctypes.CDLL(LIB_PATH)
+    lib = ctypes.CDLL(path)
     for name, (res, args) in SIGNATURES.items():
         try:
             fn = getattr(lib, name)
         except AttributeError as e:
+            if subset:
+                continue
             raise NvxLibraryError(f"{LIB_PATH} does not export {name}") from e
         fn.restype = res
         fn.argtypes = args
+    if subset:
+        lib = _SubsetLibrary(lib, path)
     want, got = header_abi_version(), lib.nvx_abi_version()
     if got != want:
         raise NvxLibraryError(f"{LIB_PATH} reports ABI version {got}, include/nvx.h declares {want}: rebuild it "

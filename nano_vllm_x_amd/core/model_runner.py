@@ -99,6 +99,10 @@ class ModelRunner:
                 torch.backends.cuda.matmul.allow_tf32 = False
                 torch.set_float32_matmul_precision("highest")
         else:
+            from .. import _lib
+            if _lib.is_subset():
+                raise _lib.NvxLibraryError("only the subset library of `make seq` is built, which has no paged-attention kernels: "
+                                           "run `make -C nano_vllm_x_amd/csrc`")
             if self._dtype_override == torch.float32:
                 raise NotImplementedError("the paged-attention kernels are built for bfloat16 and float16 only")
             self.dtype = wanted if wanted in (torch.bfloat16, torch.float16) else torch.bfloat16
