@@ -200,7 +200,7 @@ template <typename A> __device__ __forceinline__ float la_round(float v) { retur
 
 template <typename A, int RKM>      // RKM = rank / 32, the k-steps of a score product (compile time: the loops below unroll into
                                     // straight-line code, so the LDS reads of a tile run ahead of the products that use them)
-__global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
+__global__ __launch_bounds__(256, (RKM <= 8 ? 2 : 1)) void latent_attn_mfma_kernel(     // up to rank 256: two waves a SIMD
     const A* __restrict__ q, const A* __restrict__ cache, const int32_t* __restrict__ kv_indices, const int64_t* __restrict__ kv_start,
     const int32_t* __restrict__ kv_len, const int32_t* __restrict__ qo_indptr, const int32_t* __restrict__ tok_seq,
     const float* __restrict__ gate, A* __restrict__ out, int heads, int rank, int64_t n_tok, float scale) {
