@@ -42,8 +42,9 @@ typedef void* nvx_stream_t;
  *   3: float16 entry points (`*_f16`) added.
  *   4: direct-peer all-reduce (`nvx_peer_*`) and sharded sampling (`nvx_sample_shard`, `nvx_sample_pick`) added.
  *   8: layers with a 32-bit residual stream and per-sequence state (`nvx_boundary_norm`, `nvx_canon_conv`, `nvx_relu2`,
- *      `nvx_mingru_scan`) and latent attention (`nvx_latent_prep`, `nvx_latent_attn`) added. */
-#define NVX_ABI_VERSION 8
+ *      `nvx_mingru_scan`) and latent attention (`nvx_latent_prep`, `nvx_latent_attn`) added.
+ *   9: nvx_boundary_norm can apply the convolution of a decode step in the same launch. */
+#define NVX_ABI_VERSION 9
 
 /* Library identification and diagnostics. */
 int nvx_abi_version(void);
@@ -458,6 +459,8 @@ int nvx_lmhead_sample_f16(const void* w_packed, int64_t n_rows, int64_t k, const
  *     hist[hist_slot][t] = r                                             (hist_slot >= 0; slots hist_stride floats apart)
  *     x = sum_{j < n_mix} mix[j] * hist[j][t]   (n_mix > 0; hist_slot < n_mix is r itself)   else x = r
  *     x_out[t] = x;   w_pre != NULL:  y = x / sqrt(mean(x^2) + eps) * (1 + w_pre)  ->  y_f32 or y_act (exactly one)
+ *     taps != NULL (one token per sequence; width a multiple of 4, at most 8192): the convolution of nvx_canon_conv is applied
+ *     to y in the same launch -- y_act[t] = y + sum_j taps[j] * (input taps_n - 1 - j back), state[state_slot[t]] shifted by one.
  * nvx_canon_conv:  out[t] = h[t] + sum_j taps[j] * h[t - (taps_n - 1) + j]  over the tokens of t's own sequence (taps: taps_n
  *     rows of `width`);
  *     inputs before this step come from state[slot] (taps_n - 1 rows of `width`, oldest first), which is then
@@ -474,7 +477,8 @@ int nvx_lmhead_sample_f16(const void* w_packed, int64_t n_rows, int64_t k, const
  *     out[h][t] = gate[t][h] * sum_j softmax_j(scale * q[h][t] . c_j) c_j   (gate may be NULL).  rank <= 1024. */
 int nvx_boundary_norm(const void* m, int64_t m_row_stride, int fmt, const float* res, const float* w_post, float* hist,
                       int64_t hist_stride, int hist_slot, int n_mix, const float* mix, float* x_out, const float* w_pre,
-                      float* y_f32, void* y_act, int64_t n_tok, int64_t width, float eps, nvx_stream_t stream);
+                      float* y_f32, void* y_act, int64_t n_tok, int64_t width, float eps, const float* taps, int taps_n,
+                      float* state, int64_t n_slots, const int64_t* pos0, const int32_t* state_slot, nvx_stream_t stream);
 int nvx_canon_conv(const float* h, const float* taps, int taps_n, float* state, int64_t n_slots, const int32_t* tok_seq,
                    const int32_t* qo_indptr, const int64_t* pos0, const int32_t* state_slot, void* out, int fmt,
                    int64_t n_tok, int64_t n_seq, int64_t width, nvx_stream_t stream);

@@ -84,7 +84,7 @@ SIGNATURES = {
     "nvx_linear_block": (_c_i32, [_c_vp, _c_i64, _c_i64, _c_vp, _c_i64, _c_i64, _c_i32, _c_i32, _c_vp, _c_vp]),
     "nvx_peer_allreduce_norm": (_c_i32, [_c_vp, _c_vp, _c_i64, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_i64, _c_f32, _c_vp]),
     "nvx_boundary_norm": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_vp, _c_vp, _c_vp, _c_i64, _c_i32, _c_i32, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp,
-                                   _c_i64, _c_i64, _c_f32, _c_vp]),
+                                   _c_i64, _c_i64, _c_f32, _c_vp, _c_i32, _c_vp, _c_i64, _c_vp, _c_vp, _c_vp]),
     "nvx_canon_conv": (_c_i32, [_c_vp, _c_vp, _c_i32, _c_vp, _c_i64, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_i32, _c_i64, _c_i64, _c_i64, _c_vp]),
     "nvx_relu2": (_c_i32, [_c_vp, _c_vp, _c_i32, _c_i64, _c_vp]),
     "nvx_mingru_scan": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_vp, _c_i64, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_i64, _c_i64, _c_vp]),

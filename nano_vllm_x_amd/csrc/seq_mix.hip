@@ -86,7 +86,8 @@ __global__ __launch_bounds__(256) void boundary_norm_reg_kernel(
     const A* __restrict__ m, int64_t m_stride, const float* __restrict__ res, const float* __restrict__ w_post,
     float* __restrict__ hist, int64_t hist_stride, int hist_slot, int n_mix, const float* __restrict__ mix,
     float* __restrict__ x_out, const float* __restrict__ w_pre, float* __restrict__ y_f32, A* __restrict__ y_act,
-    int width, float eps) {
+    int width, float eps, const float* __restrict__ taps, int taps_n, float* __restrict__ state, const int64_t* __restrict__ pos0,
+    const int32_t* __restrict__ state_slot) {
     __shared__ float red[4];
     const int64_t t = blockIdx.x;
     const A* mr = m + t * m_stride;
@@ -125,7 +126,23 @@ __global__ __launch_bounds__(256) void boundary_norm_reg_kernel(
         const int c = (threadIdx.x + k * 256) * 4;
         if (c >= width) continue;
         const f32x4v y = v[k] * r_pre * (1.0f + *reinterpret_cast<const f32x4v*>(w_pre + c));
-        if (y_f32) *reinterpret_cast<f32x4v*>(y_f32 + row + c) = y;
+        if (taps) {
+            // one token per sequence: the convolution over the sequence's tail and the tail's shift happen here, in the one
+            // workgroup that touches this sequence (a thread reads and writes only its own channels)
+            const int slot = state_slot[t];
+            if (slot < 0) { st4(y_act + row + c, f32x4v{0.f, 0.f, 0.f, 0.f}); continue; }
+            const int hist_n = taps_n - 1;
+            const bool had = pos0[t] > 0;
+            f32x4v acc = y + *reinterpret_cast<const f32x4v*>(taps + (int64_t)hist_n * width + c) * y;
+            float* st = state + (int64_t)slot * hist_n * width + c;
+            for (int r = 0; r < hist_n; ++r) {
+                const f32x4v old = had ? *reinterpret_cast<const f32x4v*>(st + (int64_t)r * width) : f32x4v{0.f, 0.f, 0.f, 0.f};
+                acc += *reinterpret_cast<const f32x4v*>(taps + (int64_t)r * width + c) * old;
+                if (r > 0) *reinterpret_cast<f32x4v*>(st + (int64_t)(r - 1) * width) = old;
+            }
+            if (hist_n > 0) *reinterpret_cast<f32x4v*>(st + (int64_t)(hist_n - 1) * width) = y;
+            st4(y_act + row + c, acc);
+        } else if (y_f32) *reinterpret_cast<f32x4v*>(y_f32 + row + c) = y;
         else st4(y_act + row + c, y);
     }
 }
@@ -352,15 +369,18 @@ __global__ __launch_bounds__(256) void mingru_step_kernel(
 }
 
 template <typename A>
-static void launch_boundary(const void* m, int64_t m_stride, const float* res, const float* w_post, float* hist, int64_t hist_stride,
-                            int hist_slot, int n_mix, const float* mix, float* x_out, const float* w_pre, float* y_f32, void* y_act,
-                            int64_t n_tok, int width, float eps, hipStream_t s) {
+static int launch_boundary(const void* m, int64_t m_stride, const float* res, const float* w_post, float* hist, int64_t hist_stride,
+                           int hist_slot, int n_mix, const float* mix, float* x_out, const float* w_pre, float* y_f32, void* y_act,
+                           int64_t n_tok, int width, float eps, const float* taps, int taps_n, float* state, const int64_t* pos0,
+                           const int32_t* state_slot, hipStream_t s) {
     const bool vec = width % 4 == 0 && m_stride % 4 == 0 && hist_stride % 4 == 0 && nvx_aligned16(m) && nvx_aligned16(res) &&
                      nvx_aligned16(w_post) && nvx_aligned16(hist) && nvx_aligned16(x_out) && nvx_aligned16(w_pre) && nvx_aligned16(y_f32) &&
-                     nvx_aligned16(y_act);
+                     nvx_aligned16(y_act) && nvx_aligned16(taps) && nvx_aligned16(state);
+    if (taps && !(vec && width <= 8192)) return 1;     // the fused step exists in the register kernel only
 #define NVX_BOUNDARY_REG(VPT)                                                                                                         \
     hipLaunchKernelGGL((boundary_norm_reg_kernel<A, VPT>), dim3((unsigned)n_tok), dim3(256), 0, s, (const A*)m, m_stride, res, w_post, \
-                       hist, hist_stride, hist_slot, n_mix, mix, x_out, w_pre, y_f32, (A*)y_act, width, eps)
+                       hist, hist_stride, hist_slot, n_mix, mix, x_out, w_pre, y_f32, (A*)y_act, width, eps, taps, taps_n, state, pos0, \
+                       state_slot)
     if (vec && width <= 1024) NVX_BOUNDARY_REG(1);
     else if (vec && width <= 2048) NVX_BOUNDARY_REG(2);
     else if (vec && width <= 4096) NVX_BOUNDARY_REG(4);
@@ -369,6 +389,7 @@ static void launch_boundary(const void* m, int64_t m_stride, const float* res, c
         hipLaunchKernelGGL(boundary_norm_kernel<A>, dim3((unsigned)n_tok), dim3(256), 0, s, (const A*)m, m_stride, res, w_post, hist,
                            hist_stride, hist_slot, n_mix, mix, x_out, w_pre, y_f32, (A*)y_act, width, eps);
 #undef NVX_BOUNDARY_REG
+    return 0;
 }
 
 template <typename A>
@@ -416,7 +437,8 @@ using namespace NVX_NS;
 
 extern "C" int nvx_boundary_norm(const void* m, int64_t m_row_stride, int fmt, const float* res, const float* w_post, float* hist,
                                  int64_t hist_stride, int hist_slot, int n_mix, const float* mix, float* x_out, const float* w_pre,
-                                 float* y_f32, void* y_act, int64_t n_tok, int64_t width, float eps, nvx_stream_t stream) {
+                                 float* y_f32, void* y_act, int64_t n_tok, int64_t width, float eps, const float* taps, int taps_n,
+                                 float* state, int64_t n_slots, const int64_t* pos0, const int32_t* state_slot, nvx_stream_t stream) {
     NVX_REQUIRE(fmt >= 0 && fmt <= 2, NVX_EINVAL, "nvx_boundary_norm: fmt must be 0 (bfloat16), 1 (float16) or 2 (float32)");
     NVX_REQUIRE(n_tok >= 0 && width > 0 && width < (1 << 30) && m_row_stride >= width, NVX_EINVAL, "nvx_boundary_norm: bad sizes");
     if (n_tok == 0) return NVX_OK;
@@ -426,8 +448,14 @@ extern "C" int nvx_boundary_norm(const void* m, int64_t m_row_stride, int fmt, c
                 "nvx_boundary_norm: mixing needs the history buffer, the weights and this result's slot among them");
     NVX_REQUIRE(!hist || hist_stride >= n_tok * width, NVX_EINVAL, "nvx_boundary_norm: history stride smaller than a result");
     NVX_REQUIRE(!w_pre || (y_f32 != nullptr) != (y_act != nullptr), NVX_EINVAL, "nvx_boundary_norm: exactly one output for the pre-norm");
-    NVX_FMT_DISPATCH(fmt, launch_boundary<A_>(m, m_row_stride, res, w_post, hist, hist_stride, hist_slot, n_mix, mix, x_out, w_pre, y_f32,
-                                              y_act, n_tok, (int)width, eps, (hipStream_t)stream));
+    NVX_REQUIRE(!taps || (w_pre && y_act && !y_f32 && pos0 && state_slot && taps_n >= 1 && taps_n <= 64 && (state || taps_n == 1) && n_slots >= 0),
+                NVX_EINVAL, "nvx_boundary_norm: the fused convolution needs the pre-norm, y_act, pos0, state_slot and the state");
+    int unfit = 0;
+    NVX_FMT_DISPATCH(fmt, unfit = launch_boundary<A_>(m, m_row_stride, res, w_post, hist, hist_stride, hist_slot, n_mix, mix, x_out, w_pre,
+                                                      y_f32, y_act, n_tok, (int)width, eps, taps, taps_n, state, pos0, state_slot,
+                                                      (hipStream_t)stream));
+    NVX_REQUIRE(!unfit, NVX_EUNSUPPORTED, "nvx_boundary_norm: the fused convolution needs a width that is a multiple of 4, at most 8192, "
+                                          "and 16-byte aligned tensors");
     return nvx_check_launch("nvx_boundary_norm");
 }
 

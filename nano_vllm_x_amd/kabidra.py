@@ -153,6 +153,17 @@ class KabidraForCausalLM(nn.Module):
         state = md.cache.state(name) if self.config.taps > 1 else None
         return ops.canon_conv(hn, taps, state, md.layout, dtype)
 
+    def _boundary(self, y, post, x, md, dtype, pre, taps, name, **hist):
+        """A sublayer boundary and the convolution in front of the next sublayer: (new stream, that sublayer's input).  A
+        step with one token per sequence takes both in one launch; otherwise the convolution, which reads the pre-normed
+        rows of a token's predecessors, is a launch of its own."""
+        eps = self.config.eps
+        if md.layout.qo_indptr is None and ops.boundary_canon_fits(self.config.width):
+            state = md.cache.state(name) if self.config.taps > 1 else None
+            return ops.boundary_norm(y, post, eps, res=x, w_pre=pre, canon=(taps, state, md.layout), **hist)
+        x, hn = ops.boundary_norm(y, post, eps, res=x, w_pre=pre, **hist)
+        return x, self._canon(hn, taps, name, md, dtype)
+
     def forward(self, input_ids: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
         """Final-normed hidden states (tokens, width) in the activations' format.  Positions enter nowhere: the order of a
         sequence's tokens is in its state and in the causal mask."""
@@ -161,20 +172,23 @@ class KabidraForCausalLM(nn.Module):
         eps, n_layers, dtype = cfg.eps, len(self.layers), self.embed.dtype
         t = input_ids.numel()
         hist = torch.empty((n_layers + 1, t, cfg.width), dtype=torch.float32, device=input_ids.device)
-        first_pre = self.layers[0].norm1 if n_layers else self.final_norm
-        x, hn = ops.boundary_norm(F.embedding(input_ids, self.embed), self.embed_norm, eps, hist=hist, hist_slot=0, w_pre=first_pre,
-                                  pre_f32=n_layers > 0)
+        emb = F.embedding(input_ids, self.embed)
+        if n_layers == 0:
+            return ops.boundary_norm(emb, self.embed_norm, eps, w_pre=self.final_norm, pre_f32=False)[1]
+        x, h = self._boundary(emb, self.embed_norm, None, md, dtype, self.layers[0].norm1, self.layers[0].canon1, (0, "canon1"),
+                              hist=hist, hist_slot=0)
         for i, layer in enumerate(self.layers):
-            y = layer.mixer(self._canon(hn, layer.canon1, (i, "canon1"), md, dtype), md)
+            y = layer.mixer(h, md)
             post = layer.norm1b
             if layer.mlp is not None:
-                x, hn = ops.boundary_norm(y, layer.norm1b, eps, res=x, w_pre=layer.norm2)
-                y = layer.mlp(self._canon(hn, layer.canon2, (i, "canon2"), md, dtype))
+                x, h = self._boundary(y, layer.norm1b, x, md, dtype, layer.norm2, layer.canon2, (i, "canon2"))
+                y = layer.mlp(h)
                 post = layer.norm2b
-            last = i + 1 == n_layers
-            x, hn = ops.boundary_norm(y, post, eps, res=x, hist=hist, hist_slot=i + 1, mix=layer.dwa,
-                                      w_pre=self.final_norm if last else self.layers[i + 1].norm1, pre_f32=not last)
-        return hn
+            if i + 1 == n_layers:
+                return ops.boundary_norm(y, post, eps, res=x, hist=hist, hist_slot=i + 1, mix=layer.dwa, w_pre=self.final_norm,
+                                         pre_f32=False)[1]
+            nxt = self.layers[i + 1]
+            x, h = self._boundary(y, post, x, md, dtype, nxt.norm1, nxt.canon1, (i + 1, "canon1"), hist=hist, hist_slot=i + 1, mix=layer.dwa)
 
     def compute_logits(self, hidden_states: torch.Tensor) -> torch.Tensor:
         return F.linear(hidden_states, self.head)

@@ -703,12 +703,19 @@ class StepLayout:
         self.pos0, self.state_slot, self.qo_indptr, self.tok_seq = pos0, state_slot, qo_indptr, tok_seq
 
 
+def boundary_canon_fits(width: int) -> bool:
+    """Whether boundary_norm can apply the convolution of a decode step in the same launch for rows of this width."""
+    return width % 4 == 0 and width <= 8192
+
+
 def boundary_norm(m, w_post, eps: float, res=None, hist=None, hist_slot: int = -1, mix=None, w_pre=None, pre_f32: bool = True,
-                  x_out=None):
+                  x_out=None, canon=None):
     """Post-norm of a sublayer's output `m` (T, width) + residual `res` (float32) [+ weighted sum `mix` over the results
     kept in `hist` (slots, T, width), this one stored at `hist_slot`] [+ pre-norm `w_pre` of what follows].  Both norms
     are RMS norms whose stored weight is the deviation from one.  Returns (x, y): the new stream (float32) and the
-    pre-normed rows (float32 if `pre_f32`, else in m's format; None without `w_pre`)."""
+    pre-normed rows (float32 if `pre_f32`, else in m's format; None without `w_pre`).
+    `canon` = (taps, state, layout), for a step with one token per sequence: the convolution of canon_conv is applied to
+    the pre-normed rows in the same launch (state read and shifted); y is then its result, in m's format."""
     _dev(m, w_post, res, hist, mix, w_pre)
     _need(m.dim() == 2 and m.stride(1) == 1, "boundary_norm: m must be (T, width) with unit inner stride")
     t, width = m.shape
@@ -734,6 +741,23 @@ def boundary_norm(m, w_post, eps: float, res=None, hist=None, hist_slot: int = -
         _f32c(x_out, "boundary_norm: x_out")
         _need(x_out.shape == (t, width), "boundary_norm: x_out shape")
     y = None
+    taps = state = pos0 = state_slot = None
+    taps_n = n_slots = 0
+    if canon is not None:
+        taps, state, layout = canon
+        _need(w_pre is not None and layout.qo_indptr is None and layout.n_tok == t and boundary_canon_fits(width),
+              "boundary_norm: the fused convolution is for one token per sequence, a pre-norm, and a width that fits")
+        _dev(taps, state)
+        _f32c(taps, "boundary_norm: taps")
+        taps_n = taps.shape[0]
+        _need(taps.dim() == 2 and taps.shape[1] == width, "boundary_norm: taps shape")
+        if taps_n > 1:
+            _f32c(state, "boundary_norm: state")
+            _need(state.dim() == 3 and state.shape[1:] == (taps_n - 1, width), "boundary_norm: state shape")
+            n_slots = state.shape[0]
+        else:
+            state = None
+        pos0, state_slot, pre_f32 = layout.pos0, layout.state_slot, False
     if w_pre is not None:
         _f32c(w_pre, "boundary_norm: w_pre")
         _need(w_pre.numel() == width, "boundary_norm: w_pre size")
@@ -741,7 +765,8 @@ def boundary_norm(m, w_post, eps: float, res=None, hist=None, hist_slot: int = -
     lib = _lib.load()
     _lib.check(lib.nvx_boundary_norm(_ptr(m), m.stride(0), _fmt(m), _ptr(res), _ptr(w_post), _ptr(hist), hist_stride, hist_slot, n_mix,
                                      _ptr(mix), _ptr(x_out), _ptr(w_pre), _ptr(y) if (y is not None and pre_f32) else None,
-                                     _ptr(y) if (y is not None and not pre_f32) else None, t, width, float(eps), _stream()),
+                                     _ptr(y) if (y is not None and not pre_f32) else None, t, width, float(eps), _ptr(taps), taps_n,
+                                     _ptr(state), n_slots, _ptr(pos0), _ptr(state_slot), _stream()),
                "nvx_boundary_norm")
     return x_out, y
 

@@ -60,7 +60,7 @@ _DEFS = {
     # layers with a float32 residual stream, per-sequence state and latent attention; the step's layout travels as its four
     # tensors (qo_indptr and tok_seq absent: one token per sequence)
     "boundary_norm": "(Tensor m, Tensor w_post, float eps, Tensor? res, Tensor(a!)? hist, int hist_slot, Tensor? mix, Tensor? w_pre, "
-                     "bool pre_f32) -> (Tensor, Tensor?)",
+                     "bool pre_f32, Tensor? taps, Tensor(b!)? state, Tensor? pos0, Tensor? state_slot) -> (Tensor, Tensor?)",
     "canon_conv": "(Tensor h, Tensor taps, Tensor(a!) state, Tensor pos0, Tensor state_slot, Tensor? qo_indptr, Tensor? tok_seq, "
                   "ScalarType dtype) -> Tensor",
     "relu2": "(Tensor x) -> Tensor",
@@ -201,8 +201,9 @@ def _layout(n_tok, pos0, state_slot, qo_indptr, tok_seq):
     return ops.StepLayout(n_tok, n_seq, pos0, state_slot, qo_indptr, tok_seq)
 
 
-def _boundary_norm(m, w_post, eps, res, hist, hist_slot, mix, w_pre, pre_f32):
-    return ops.boundary_norm(m, w_post, eps, res=res, hist=hist, hist_slot=hist_slot, mix=mix, w_pre=w_pre, pre_f32=pre_f32)
+def _boundary_norm(m, w_post, eps, res, hist, hist_slot, mix, w_pre, pre_f32, taps, state, pos0, state_slot):
+    canon = None if taps is None else (taps, state, _layout(m.shape[0], pos0, state_slot, None, None))
+    return ops.boundary_norm(m, w_post, eps, res=res, hist=hist, hist_slot=hist_slot, mix=mix, w_pre=w_pre, pre_f32=pre_f32, canon=canon)
 
 
 def _canon_conv(h, taps, state, pos0, state_slot, qo_indptr, tok_seq, dtype):

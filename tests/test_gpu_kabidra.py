@@ -159,6 +159,34 @@ def test_canon_conv_continues_over_cuts_of_every_length(taps):
     assert torch.allclose(out, ko.canon(fresh, k), atol=1e-5), "a sequence at position 0 must not read the slot's old tail"
 
 
+@pytest.mark.parametrize("taps,width", [(1, 8), (2, 1028), (4, 96), (5, 2052)])
+def test_boundary_norm_with_the_convolution_of_a_decode_step(taps, width):
+    """One token per sequence, step after step: the fused launch against norm + convolution over the whole history.  The
+    second sequence starts two steps later in a slot that holds another sequence's tail."""
+    from nano_vllm_x_amd import ops
+    g = torch.Generator().manual_seed(taps)
+    steps, eps = 7, 1e-4
+    k = torch.randn(width, taps, generator=g)
+    w_post, w_pre = 0.2 * torch.randn(width, generator=g), 0.2 * torch.randn(width, generator=g)
+    m = torch.randn(2, steps, width, generator=g)
+    res = torch.randn(2, steps, width, generator=g)
+    start = [0, 2]
+    want = []
+    for b in range(2):
+        x = res[b, start[b]:] + ko.norm_zero_centred(m[b, start[b]:], w_post, eps)
+        want.append(ko.canon(ko.norm_zero_centred(x, w_pre, eps), k))
+    state = torch.full((3, taps - 1, width), 9.0).cuda() if taps > 1 else None
+    kt = k.t().contiguous().cuda()
+    for s in range(steps):
+        live = [b for b in range(2) if s >= start[b]]
+        lay = _layout(ops, [1] * len(live), [s - start[b] for b in live], [2 - b for b in live], decode=True)
+        x, y = ops.boundary_norm(torch.stack([m[b, s] for b in live]).cuda(), w_post.cuda(), eps, res=torch.stack([res[b, s] for b in live]).cuda(),
+                                 w_pre=w_pre.cuda(), canon=(kt, state, lay))
+        for i, b in enumerate(live):
+            assert torch.allclose(y[i].cpu(), want[b][s - start[b]], atol=2e-5), (b, s)
+            assert torch.allclose(x[i].cpu(), res[b, s] + ko.norm_zero_centred(m[b, s], w_post, eps), atol=1e-5)
+
+
 @pytest.mark.parametrize("width", [24, 64, 130])
 def test_mingru_scan_over_cuts_and_round_borders(width):
     """The scan works in rounds of 128 tokens: lengths around one and several rounds, steps of one token, a long memory
