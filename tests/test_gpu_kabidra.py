@@ -125,7 +125,7 @@ def _layout(ops, lens, pos0, slots, decode=False):
     return ops.StepLayout(int(qo[-1]), n, p, s, torch.from_numpy(qo).cuda(), torch.from_numpy(tok).cuda())
 
 
-@pytest.mark.parametrize("taps", [1, 2, 4, 6])
+@pytest.mark.parametrize("taps", [1, 2, 4, 6, 10])
 def test_canon_conv_continues_over_cuts_of_every_length(taps):
     """Two sequences in slots that are not in order, cut into steps of 1, 2, taps - 1, taps and more tokens; a third
     sequence later takes over a used slot and must not see what is left there."""
