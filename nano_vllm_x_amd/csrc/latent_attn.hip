@@ -203,11 +203,15 @@ template <typename A, int RKM>      // RKM = rank / 32, the k-steps of a score p
 __global__ __launch_bounds__(256, (RKM <= 8 ? 2 : 1)) void latent_attn_mfma_kernel(     // up to rank 256: two waves a SIMD
     const A* __restrict__ q, const A* __restrict__ cache, const int32_t* __restrict__ kv_indices, const int64_t* __restrict__ kv_start,
     const int32_t* __restrict__ kv_len, const int32_t* __restrict__ qo_indptr, const int32_t* __restrict__ tok_seq,
-    const float* __restrict__ gate, A* __restrict__ out, int heads, int rank, int64_t n_tok, float scale) {
+    const float* __restrict__ gate, A* __restrict__ out, int heads, int rank, int64_t n_tok, float scale, int skip_groups) {
     extern __shared__ float lds[];
     constexpr int NB2 = RKM;                   // pairs of 16-column blocks = rank / 32
     constexpr int steps = RKM;
     const int64_t t = blockIdx.x;
+    if (skip_groups) {                         // tokens whose group of four lies in one sequence belong to the tile kernel below
+        const int64_t g0 = t & ~(int64_t)3;
+        if (g0 + 3 < n_tok && tok_seq[g0] == tok_seq[g0 + 3]) return;
+    }
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, l16 = lane & 15, quarter = lane >> 4;
     const int head = blockIdx.y * 16 + l16;
     const int b = tok_seq ? tok_seq[t] : (int)t;
@@ -359,6 +363,136 @@ __global__ __launch_bounds__(256, (RKM <= 8 ? 2 : 1)) void latent_attn_mfma_kern
     }
 }
 
+// ---- prefill: four query tokens of one sequence share every key tile -----------------------------------------------------
+// Workgroup = tokens 4g .. 4g+3 of the step's token list, if they belong to one sequence (other groups return at once and
+// are served by the kernel above, launched with skip_groups); wave w owns token 4g + w and all of its keys.  A tile's rows
+// are fetched once for the four tokens -- each wave brings a quarter of the k-steps, one tile ahead, into the other of
+// two LDS buffers -- so the cache is read a quarter as often, no merge is needed at the end, and the score product takes
+// its A operand from LDS.  One barrier per tile.  The arithmetic per tile is the kernel's above.
+template <typename A, int RKM>
+__global__ __launch_bounds__(256, (RKM <= 8 ? 2 : 1)) void latent_attn_mfma_tile_kernel(
+    const A* __restrict__ q, const A* __restrict__ cache, const int32_t* __restrict__ kv_indices, const int64_t* __restrict__ kv_start,
+    const int32_t* __restrict__ kv_len, const int32_t* __restrict__ qo_indptr, const int32_t* __restrict__ tok_seq,
+    const float* __restrict__ gate, A* __restrict__ out, int heads, int rank, int64_t n_tok, float scale) {
+    extern __shared__ float lds[];
+    constexpr int NB2 = RKM, MY = (RKM + 3) / 4;
+    const int64_t t0 = (int64_t)blockIdx.x * 4;
+    if (t0 + 3 >= n_tok) return;
+    const int b = tok_seq[t0];
+    if (tok_seq[t0 + 3] != b) return;
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, l16 = lane & 15, quarter = lane >> 4;
+    const int64_t t = t0 + wv;
+    const int head = blockIdx.y * 16 + l16;
+    const int64_t q0 = qo_indptr[b];
+    const int64_t first = (int64_t)kv_len[b] - (qo_indptr[b + 1] - q0) - q0 + 1;      // keys of token t: first + t
+    const int64_t n_keys = first + t, n_keys_max = first + t0 + 3;
+    const int32_t* idx = kv_indices + kv_start[b];
+    const int row_elems = rank + LA_PAD;
+    uint16_t* buf0 = reinterpret_cast<uint16_t*>(lds);
+    uint16_t* buf1 = buf0 + 16 * row_elems;
+
+    nvx_u32x4 qb[RKM];
+#pragma unroll
+    for (int ks = 0; ks < RKM; ++ks) {
+        qb[ks] = nvx_u32x4{0u, 0u, 0u, 0u};
+        if (head < heads) qb[ks] = *reinterpret_cast<const nvx_u32x4*>(q + ((int64_t)head * n_tok + t) * rank + 32 * ks + 8 * quarter);
+    }
+    nvx_f32x4 o_acc[2 * NB2];
+#pragma unroll
+    for (int i = 0; i < 2 * NB2; ++i) o_acc[i] = nvx_f32x4{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;
+
+    const int64_t n_tiles = (n_keys_max + 15) >> 4;
+    nvx_u32x4 a_nxt[MY];
+    auto slot_of = [&](int64_t j) {
+        const int64_t key = j * 16 + l16;
+        return idx[key < n_keys_max ? key : 0];
+    };
+    auto fetch = [&](int slot) {
+        const A* row = cache + (int64_t)slot * rank;
+#pragma unroll
+        for (int i = 0; i < MY; ++i)
+            if (wv + 4 * i < RKM) a_nxt[i] = *reinterpret_cast<const nvx_u32x4*>(row + 32 * (wv + 4 * i) + 8 * quarter);
+    };
+    auto park = [&](uint16_t* buf) {
+#pragma unroll
+        for (int i = 0; i < MY; ++i)
+            if (wv + 4 * i < RKM) *reinterpret_cast<nvx_u32x4*>(buf + l16 * row_elems + 32 * (wv + 4 * i) + 8 * quarter) = a_nxt[i];
+    };
+    int slot_nxt = 0;
+    fetch(slot_of(0));
+    if (1 < n_tiles) slot_nxt = slot_of(1);
+    park(buf0);
+    __syncthreads();
+    for (int64_t j = 0; j < n_tiles; ++j) {
+        const uint16_t* tile = (j & 1) ? buf1 : buf0;
+        if (j + 1 < n_tiles) fetch(slot_nxt);
+        if (j + 2 < n_tiles) slot_nxt = slot_of(j + 2);
+        if (j * 16 < n_keys) {                                   // (a last tile may hold only keys of the later tokens)
+            nvx_f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < RKM; ++ks) {
+                const nvx_u32x4 a = *reinterpret_cast<const nvx_u32x4*>(tile + l16 * row_elems + 32 * ks + 8 * quarter);
+                sacc = la_mfma32<A>(a, qb[ks], sacc);
+            }
+            float sv[4], mx = -INFINITY;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                sv[r] = (j * 16 + 4 * quarter + r) < n_keys ? sacc[r] * scale : -INFINITY;
+                mx = fmaxf(mx, sv[r]);
+            }
+            mx = fmaxf(mx, xor16(mx));
+            mx = fmaxf(mx, xor32(mx));
+            const float m_new = fmaxf(m_run, mx);
+            const float alpha = __expf(m_run - m_new);
+            const bool rescale = __any(alpha != 1.0f);
+            m_run = m_new;
+            l_run *= alpha;
+            float p[4], ph[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                p[r] = __expf(sv[r] - m_new);
+                l_run += p[r];
+                ph[r] = la_round<A>(p[r]);
+            }
+            const uint2 p_hi = make_uint2(la_pack2<A>(ph[0], ph[1]), la_pack2<A>(ph[2], ph[3]));
+            const uint2 p_lo = make_uint2(la_pack2<A>(p[0] - ph[0], p[1] - ph[1]), la_pack2<A>(p[2] - ph[2], p[3] - ph[3]));
+            const uint32_t* tile32 = reinterpret_cast<const uint32_t*>(tile);
+#pragma unroll
+            for (int b2 = 0; b2 < NB2; ++b2) {
+                uint32_t d[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) d[r] = tile32[((4 * quarter + r) * row_elems + 32 * b2) / 2 + l16];
+                const uint2 even = make_uint2((d[0] & 0xffffu) | (d[1] << 16), (d[2] & 0xffffu) | (d[3] << 16));
+                const uint2 odd = make_uint2((d[0] >> 16) | (d[1] & 0xffff0000u), (d[2] >> 16) | (d[3] & 0xffff0000u));
+                if (rescale) {
+                    o_acc[2 * b2] *= alpha;
+                    o_acc[2 * b2 + 1] *= alpha;
+                }
+                o_acc[2 * b2] = la_mfma16<A>(even, p_hi, o_acc[2 * b2]);
+                o_acc[2 * b2] = la_mfma16<A>(even, p_lo, o_acc[2 * b2]);
+                o_acc[2 * b2 + 1] = la_mfma16<A>(odd, p_hi, o_acc[2 * b2 + 1]);
+                o_acc[2 * b2 + 1] = la_mfma16<A>(odd, p_lo, o_acc[2 * b2 + 1]);
+            }
+        }
+        if (j + 1 < n_tiles) park((j & 1) ? buf0 : buf1);        // the buffer whose readers passed the barrier before
+        __syncthreads();
+    }
+    float l_tot = l_run + xor16(l_run);
+    l_tot += xor32(l_tot);
+    if (head >= heads) return;
+    const float f = (gate ? gate[t * heads + head] : 1.0f) / l_tot;
+    A* orow = out + ((int64_t)head * n_tok + t) * rank;
+#pragma unroll
+    for (int b2 = 0; b2 < NB2; ++b2) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int c = 32 * b2 + 2 * (4 * quarter + r);
+            *reinterpret_cast<uint32_t*>(orow + c) = la_pack2<A>(o_acc[2 * b2][r] * f, o_acc[2 * b2 + 1][r] * f);
+        }
+    }
+}
+
 template <typename A>
 static void launch_prep(const void* x, int64_t x_stride, const float* w_q, const float* w_kv, float eps, const int64_t* slots, void* cq,
                         void* cache, int64_t n_slots, float* gate, int64_t n_tok, int q_rank, int kv_rank, int heads, hipStream_t s) {
@@ -377,9 +511,18 @@ static void launch_attn(const void* q, const void* cache, const int32_t* kv_indi
             const size_t tiles = (size_t)4 * 16 * (rank + LA_PAD) * 2, merge = (size_t)2 * (8 * steps + 2) * 64 * 4;
             const size_t lds = tiles > merge ? tiles : merge;
             const dim3 grid((unsigned)n_tok, (unsigned)((heads + 15) / 16));
+            // a ragged step: groups of four tokens inside one sequence go to the tile-sharing kernel, the rest stay here
+            const int grouped = qo_indptr != nullptr && n_tok >= 4;
+            const dim3 grid4((unsigned)(n_tok / 4), grid.y);
+            const size_t lds4 = (size_t)2 * 16 * (rank + LA_PAD) * 2;
 #define NVX_LA_MFMA(RKM)                                                                                                            \
-    hipLaunchKernelGGL((latent_attn_mfma_kernel<A, RKM>), grid, dim3(256), lds, s, (const A*)q, (const A*)cache, kv_indices, kv_start, \
-                       kv_len, qo_indptr, tok_seq, gate, (A*)out, heads, rank, n_tok, scale)
+    do {                                                                                                                            \
+        if (grouped)                                                                                                                \
+            hipLaunchKernelGGL((latent_attn_mfma_tile_kernel<A, RKM>), grid4, dim3(256), lds4, s, (const A*)q, (const A*)cache,       \
+                               kv_indices, kv_start, kv_len, qo_indptr, tok_seq, gate, (A*)out, heads, rank, n_tok, scale);           \
+        hipLaunchKernelGGL((latent_attn_mfma_kernel<A, RKM>), grid, dim3(256), lds, s, (const A*)q, (const A*)cache, kv_indices,      \
+                           kv_start, kv_len, qo_indptr, tok_seq, gate, (A*)out, heads, rank, n_tok, scale, grouped);                 \
+    } while (0)
             switch (steps) {
                 case 1: NVX_LA_MFMA(1); break;
                 case 2: NVX_LA_MFMA(2); break;
