@@ -508,3 +508,20 @@ def test_preempted_sequence_starts_again_from_an_empty_state(tmp_path):
     for i, p in prompts.items():
         assert out[i] == oracle_greedy(w, cfg, p, 14), i
     eng.shutdown()
+
+
+def test_command_line_generates_what_the_restatement_does(tmp_path):
+    import subprocess
+    import sys
+    cfg = make_cfg([GRU, ATT], vocab=90)
+    path = model_dir(tmp_path, cfg)
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, "-m", "nano_vllm_x_amd", "--model", path, "--prompt-ids", "5,17,3,44", "--prompt-ids", "8",
+                          "--max-new-tokens", "6", "--dtype", "float32", "--kv-cache-size", "128", "--context-len", "64", "--max-bs", "2",
+                          "--seed", "3"], cwd=root, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr[-2000:]
+    lines = [json.loads(x) for x in out.stdout.splitlines() if x.startswith("{")]
+    w = weights_of(cfg, 3)
+    assert [x["prompt"] for x in lines] == [[5, 17, 3, 44], [8]]
+    for x in lines:
+        assert x["generated_ids"] == oracle_greedy(w, cfg, x["prompt"], 6)
