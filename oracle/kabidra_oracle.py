@@ -87,7 +87,7 @@ def sub(w: dict, prefix: str) -> dict:
 
 def forward(w: dict, cfg: dict, tokens, dtype=torch.float32, layers_out=None) -> torch.Tensor:
     """Logits (tokens, vocab) of one whole sequence.  `w`: name -> tensor; `layers_out`, if a list, receives every
-    layer's result (before the depth average)."""
+    layer's result (before the weighted sum over the depth)."""
     w = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in w.items()}
     eps = cfg["norm"]["eps"]
     x = norm_zero_centred(w["embed"][torch.as_tensor(tokens)], w["embed.norm"], eps)
