@@ -331,6 +331,22 @@ def test_other_sizes_one_head_no_feed_forward_equal_ranks(tmp_path):
         eng.shutdown()
 
 
+def test_sizes_that_fit_no_vector_width(tmp_path):
+    """Odd width, odd recurrence width, ranks and head sizes that are multiples of nothing: every kernel's plain path."""
+    att = {"type": "latent_attention", "mixer": {"heads": 2, "dim": 5, "vdim": 7, "q_rank": 11, "kv_rank": 13, "scale": 0.7},
+           "mlp": {"kind": "dense", "ff": 19}}
+    gru = {"type": "mingru", "mixer": {"width": 25}, "mlp": {"kind": "dense", "ff": 9}}
+    cfg = make_cfg([gru, att, att, gru], width=30, vocab=23, taps=4)
+    cfg["width"] = 27
+    toks = tokens(150, 23, 8)
+    want = ko.forward(weights_of(cfg, 4), cfg, toks, torch.float64)
+    for dtype, tol in (("float32", F32_TOL), ("bfloat16", 0.15)):
+        eng = make_engine(model_dir(tmp_path, cfg, name=dtype), dtype=dtype, seed=4)
+        got = replay(eng, {"a": toks}, [[("a", 100)], [("a", 3)]] + [[("a", 1)]] * 47)["a"]
+        close(got, want, tol, dtype)
+        eng.shutdown()
+
+
 def test_unequal_requests_in_one_batch_and_slots_that_change_hands(tmp_path):
     """Four live requests at most, in a pool that holds less than all of them: portions beside single tokens, requests
     that end and whose token slots and state slot go to the next one.  Every request against itself alone."""
