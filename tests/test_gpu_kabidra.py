@@ -492,6 +492,30 @@ def test_decode_steps_replay_a_captured_graph(tmp_path, dtype):
         assert got == run(True)[0]
 
 
+def test_decode_steps_queued_ahead_give_the_same_tokens(tmp_path):
+    """run_ahead: decode step N+1 is queued before step N's ids reach the host; the rows' state slots and slot lists of both
+    steps are in flight at once."""
+    from nano_vllm_x_amd.core.common import SamplingParams
+    from nano_vllm_x_amd.core.engine import Engine
+    cfg = make_cfg([GRU, ATT, GRU])
+    path = model_dir(tmp_path, cfg)
+    eng = Engine(model=path, gpu_memory_utilization=0.5, max_bs=3, enforce_eager=False, context_len=128, kv_cache_size=300, dtype="float32",
+                 seed=8, run_ahead=True)
+    prompts = {f"r{k}": tokens(n, cfg["vocab"], 60 + k) for k, n in enumerate([7, 19, 3])}
+    new = {"r0": 21, "r1": 9, "r2": 15}
+    for i, p in prompts.items():
+        eng.add_sequence(i, list(p), SamplingParams(temperature=0.0, ignore_eos=True, max_new_tokens=new[i]))
+    out = {i: [] for i in prompts}
+    while eng.has_unfinished_sequences() or eng.step_in_flight:
+        for o in eng.step_overlapped():
+            out[o.seq_id].append(o.new_token_id)
+    assert eng.ahead_steps > 5
+    w = weights_of(cfg, 8)
+    for i, p in prompts.items():
+        assert out[i] == oracle_greedy(w, cfg, p, new[i]), i
+    eng.shutdown()
+
+
 def test_generate_entry_point(tmp_path):
     from nano_vllm_x_amd import LLM, SamplingParams
     cfg = make_cfg([ATT, GRU], vocab=300)
