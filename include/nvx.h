@@ -44,7 +44,7 @@ typedef void* nvx_stream_t;
  *   8: layers with a 32-bit residual stream and per-sequence state (`nvx_boundary_norm`, `nvx_canon_conv`, `nvx_relu2`,
  *      `nvx_mingru_scan`) and latent attention (`nvx_latent_prep`, `nvx_latent_attn`) added.
  *   9: nvx_boundary_norm can apply the convolution of a decode step in the same launch. */
-#define NVX_ABI_VERSION 9
+#define NVX_ABI_VERSION 10
 
 /* Library identification and diagnostics. */
 int nvx_abi_version(void);
@@ -492,6 +492,91 @@ int nvx_latent_prep(const void* x, int64_t x_row_stride, int fmt, const float* w
 int nvx_latent_attn(const void* q, const void* cache, int fmt, const int32_t* kv_indices, const int64_t* kv_start,
                     const int32_t* kv_len, const int32_t* qo_indptr, const int32_t* tok_seq, const float* gate, void* out,
                     int64_t heads, int64_t rank, int64_t n_tok, float scale, nvx_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------
+ * More layers for the same kind of stack (float32 stream, per-sequence state, ragged batches as above; `fmt` as above).
+ *
+ * nvx_gated_residual_norm, per token t:
+ *     r = y[t], or with y2: r = (y[t] / rms(y[t]) * w_y + y2[t] / rms(y2[t]) * w_y2) / 2      (rms over the whole row, with eps)
+ *     gate != NULL: r *= sigmoid(gate[t] + gate_bias)   (gate_bias may be NULL);   x[t] += mult * r   (y == NULL: x unchanged)
+ *     w_norm != NULL: h_out[t] = x[t] with each of `groups` consecutive slices divided by sqrt(mean(slice^2) + eps), times w_norm.
+ * nvx_head_norm_gate:  out[t][h] = o[t][h] / rms(o[t][h]) * w * G   per head of vdim values; w has heads * vdim entries, or vdim
+ *     shared by the heads (w_shared); kind 0: G = 1, 1: G = sigmoid(gate), 2: G = gate * sigmoid(gate)  (gate laid out as out).
+ * nvx_short_conv_silu:  out[t][c] = silu(sum_j w[j][c] * x[t - (taps_n - 1) + j][c]) over t's own sequence (w: taps_n rows of
+ *     `channels`); inputs before this step come from state[slot] (taps_n - 1 rows, oldest first), which is then replaced by the
+ *     sequence's last taps_n - 1 inputs; inputs before the sequence's start are zero.
+ * nvx_token_shift_mix:  out[m][t] = h[t] + (h[t-1] - h[t]) * mu[m]  for m < n_mix (out: n_mix blocks of n_tok rows); the
+ *     predecessor of a step's first token is state[slot] (zeros at position 0), which then takes the sequence's last row.
+ * nvx_mlstm_scan:  x[t] holds q at q_off, k at k_off (heads * dim) and v at v_off (heads * vdim); gates[t] = [i | f] pre-activations
+ *     (float32, heads each; gate_bias likewise).  i' = cap tanh((i + b_i) / cap), f' = logsigmoid(cap tanh((f + b_f) / cap));
+ *     m <- max(f' + m_old, i');  S <- e^(f' + m_old - m) S + e^(i' - m) k v^T;  n likewise with k;
+ *     out[t] = S^T q dim^(-1/2) / (max(|n . q dim^(-1/2)|, e^(-m)) + 1e-6)   (float32, heads * vdim).  S (slots, heads, dim, vdim),
+ *     N (slots, heads, dim), M (slots, heads) are continued and written back; all start from zero.  dim <= 512.
+ * nvx_delta_scan:  x[t] holds q at q_off, k at k_off (kv_heads * dim) and v at v_off (heads * vdim); ab[t] = [a | b] (float32, heads
+ *     each).  q, k <- unit length per head (x / sqrt(sum x^2 + 1e-6)), q also times dim^(-1/2);  g = exp(-exp(a_log) softplus(a +
+ *     dt_bias)), beta = sigmoid(b);  S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  out[t] = S^T q.  Head h reads q/k head
+ *     h / (heads / kv_heads).  dim <= 512.
+ * nvx_rwkv_scan:  r, k, v: (n_tok, heads * dim), rows rkv_stride apart; w = exp(-exp(wlog[t] + w0)) per key channel; bonus (heads,
+ *     dim);  out[t] = (S + diag(bonus) k v^T)^T r;  S <- diag(w) S + k v^T.   S (slots, heads, dim, dim).  dim <= 256.
+ * nvx_rope_vnorm_store:  x[t] = [q (heads * dim) | k (kv_heads * dim) | v (kv_heads * vdim)].  The first rot_dims of every q and k
+ *     head are rotated in pairs (i, i + rot_dims / 2) by the angle positions[t] * freq[i]: (u, v) -> mag * (u cos - v sin, v cos
+ *     + u sin).  q_out[t] takes the rotated q, k_cache[slots[t]] the rotated k, v_cache[slots[t]] each value head divided by its
+ *     root mean square (with eps).  A negative slot stores nothing.
+ * nvx_softcap_attn:  token t of sequence b attends over the rows at slots kv_indices[kv_start[b] + j], j <= kv_len[b] - q_len[b] +
+ *     (t - qo_indptr[b]):  s_j = scale * q . k_j,  s_j <- cap tanh(s_j / cap) (cap > 0),  out = softmax(s) V.  Query head h reads
+ *     key/value head h / (heads / kv_heads).  q (n_tok, heads * dim), k_cache (slots, kv_heads * dim), v_cache (slots, kv_heads *
+ *     vdim), out (n_tok, heads * vdim).
+ * nvx_moe_route:  idx[t][k], wts[t][k] = the expert with the k-th largest logit of token t (ties: the lower id) and the sigmoid
+ *     of that logit.
+ * Expert e:  g = min(W_gate x, limit), u = clamp(W_up x, -limit, limit), y = g sigmoid(alpha g) (u + 1), result W_down y, with
+ *     w_gu (experts, 2 ff, width) = rows [gate | up] and w_d (experts, width, ff).
+ * nvx_moe_expert_rows:  out[t] = sum_k expert_idx[t][k](wts[t][k] * h[t]), a workgroup per token (width <=
+ *     nvx_moe_expert_rows_max_width(ff)).
+ * nvx_moe_scatter_rows:  xs[dst[r]] = wts[r] * h[r / top] for every (token, choice) pair r.
+ * nvx_moe_glu:  y[r][j] = the expert's activation of (gu[r][j], gu[r][ff + j]).
+ * nvx_moe_gather_rows:  out[t] = sum_k ys[dst[t * top + k]]. */
+int nvx_gated_residual_norm(const void* y, int64_t y_stride, const void* y2, int64_t y2_stride, const float* w_y,
+                            const float* w_y2, const void* gate, int64_t gate_stride, const float* gate_bias, int fmt,
+                            float mult, float* x, const float* w_norm, int groups, float eps, void* h_out, int64_t n_tok,
+                            int64_t width, nvx_stream_t stream);
+int nvx_head_norm_gate(const float* o, const float* w, int w_shared, const void* gate, int64_t gate_stride, int kind, int fmt,
+                       float eps, void* out, int64_t n_tok, int64_t heads, int64_t vdim, nvx_stream_t stream);
+int nvx_short_conv_silu(const void* x, int64_t x_stride, int fmt, const float* w, int taps_n, float* state, int64_t n_slots,
+                        const int32_t* tok_seq, const int32_t* qo_indptr, const int64_t* pos0, const int32_t* state_slot,
+                        void* out, int64_t n_tok, int64_t n_seq, int64_t channels, nvx_stream_t stream);
+int nvx_token_shift_mix(const void* h, int64_t h_stride, int fmt, const float* mu, int n_mix, float* state, int64_t n_slots,
+                        const int32_t* tok_seq, const int32_t* qo_indptr, const int64_t* pos0, const int32_t* state_slot,
+                        void* out, int64_t n_tok, int64_t n_seq, int64_t width, nvx_stream_t stream);
+int nvx_mlstm_scan(const void* x, int64_t x_stride, int fmt, int64_t q_off, int64_t k_off, int64_t v_off, const float* gates,
+                   const float* gate_bias, float cap, float* S, float* N, float* M, int64_t n_slots, const int32_t* qo_indptr,
+                   const int64_t* pos0, const int32_t* state_slot, float* out, int64_t n_tok, int64_t n_seq, int64_t heads,
+                   int64_t dim, int64_t vdim, nvx_stream_t stream);
+int nvx_delta_scan(const void* x, int64_t x_stride, int fmt, int64_t q_off, int64_t k_off, int64_t v_off, const float* ab,
+                   const float* a_log, const float* dt_bias, float* S, int64_t n_slots, const int32_t* qo_indptr,
+                   const int64_t* pos0, const int32_t* state_slot, float* out, int64_t n_tok, int64_t n_seq, int64_t heads,
+                   int64_t kv_heads, int64_t dim, int64_t vdim, nvx_stream_t stream);
+int nvx_rwkv_scan(const void* r, const void* k, const void* v, int64_t rkv_stride, int fmt, const float* wlog, const float* w0,
+                  const float* bonus, float* S, int64_t n_slots, const int32_t* qo_indptr, const int64_t* pos0,
+                  const int32_t* state_slot, float* out, int64_t n_tok, int64_t n_seq, int64_t heads, int64_t dim,
+                  nvx_stream_t stream);
+int nvx_rope_vnorm_store(const void* x, int64_t x_stride, int fmt, const int64_t* positions, const double* freq, float mag,
+                         int rot_dims, float eps, const int64_t* slots, void* q_out, void* k_cache, void* v_cache,
+                         int64_t n_slots, int64_t n_tok, int64_t heads, int64_t kv_heads, int64_t dim, int64_t vdim,
+                         nvx_stream_t stream);
+int nvx_softcap_attn(const void* q, const void* k_cache, const void* v_cache, int fmt, const int32_t* kv_indices,
+                     const int64_t* kv_start, const int32_t* kv_len, const int32_t* qo_indptr, const int32_t* tok_seq,
+                     float scale, float cap, void* out, int64_t n_tok, int64_t heads, int64_t kv_heads, int64_t dim, int64_t vdim,
+                     nvx_stream_t stream);
+int nvx_moe_route(const float* logits, int64_t n_tok, int64_t n_exp, int64_t top, int32_t* idx, float* wts, nvx_stream_t stream);
+int64_t nvx_moe_expert_rows_max_width(int64_t ff);
+int nvx_moe_expert_rows(const void* h, int64_t h_stride, int fmt, const int32_t* idx, const float* wts, int64_t top,
+                        const void* w_gu, const void* w_d, int64_t n_exp, float limit, float alpha, void* out, int64_t n_tok,
+                        int64_t width, int64_t ff, nvx_stream_t stream);
+int nvx_moe_scatter_rows(const void* h, int64_t h_stride, int fmt, const float* wts, const int64_t* dst, int64_t top, void* xs,
+                         int64_t n_tok, int64_t width, nvx_stream_t stream);
+int nvx_moe_glu(const void* gu, int fmt, float limit, float alpha, void* y, int64_t rows, int64_t ff, nvx_stream_t stream);
+int nvx_moe_gather_rows(const void* ys, int fmt, const int64_t* dst, int64_t top, void* out, int64_t n_tok, int64_t width,
+                        nvx_stream_t stream);
 
 #ifdef __cplusplus
 }

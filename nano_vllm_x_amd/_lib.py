@@ -92,6 +92,30 @@ SIGNATURES = {
                                  _c_i64, _c_vp]),
     "nvx_latent_attn": (_c_i32, [_c_vp, _c_vp, _c_i32, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_i64, _c_i64, _c_f32,
                                  _c_vp]),
+    "nvx_gated_residual_norm": (_c_i32, [_c_vp, _c_i64, _c_vp, _c_i64, _c_vp, _c_vp, _c_vp, _c_i64, _c_vp, _c_i32, _c_f32, _c_vp, _c_vp, _c_i32,
+                                         _c_f32, _c_vp, _c_i64, _c_i64, _c_vp]),
+    "nvx_head_norm_gate": (_c_i32, [_c_vp, _c_vp, _c_i32, _c_vp, _c_i64, _c_i32, _c_i32, _c_f32, _c_vp, _c_i64, _c_i64, _c_i64, _c_vp]),
+    "nvx_short_conv_silu": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_vp, _c_i32, _c_vp, _c_i64, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_i64,
+                                     _c_i64, _c_vp]),
+    "nvx_token_shift_mix": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_vp, _c_i32, _c_vp, _c_i64, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_i64,
+                                     _c_i64, _c_vp]),
+    "nvx_mlstm_scan": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_i64, _c_i64, _c_i64, _c_vp, _c_vp, _c_f32, _c_vp, _c_vp, _c_vp, _c_i64, _c_vp, _c_vp,
+                                _c_vp, _c_vp, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_vp]),
+    "nvx_delta_scan": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_i64, _c_i64, _c_i64, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_vp, _c_vp, _c_vp, _c_vp,
+                                _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_vp]),
+    "nvx_rwkv_scan": (_c_i32, [_c_vp, _c_vp, _c_vp, _c_i64, _c_i32, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64,
+                               _c_i64, _c_i64, _c_i64, _c_vp]),
+    "nvx_rope_vnorm_store": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_vp, _c_vp, _c_f32, _c_i32, _c_f32, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_i64,
+                                      _c_i64, _c_i64, _c_i64, _c_i64, _c_vp]),
+    "nvx_softcap_attn": (_c_i32, [_c_vp, _c_vp, _c_vp, _c_i32, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_f32, _c_f32, _c_vp, _c_i64, _c_i64, _c_i64,
+                                  _c_i64, _c_i64, _c_vp]),
+    "nvx_moe_route": (_c_i32, [_c_vp, _c_i64, _c_i64, _c_i64, _c_vp, _c_vp, _c_vp]),
+    "nvx_moe_expert_rows_max_width": (_c_i64, [_c_i64]),
+    "nvx_moe_expert_rows": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_vp, _c_vp, _c_i64, _c_vp, _c_vp, _c_i64, _c_f32, _c_f32, _c_vp, _c_i64, _c_i64,
+                                     _c_i64, _c_vp]),
+    "nvx_moe_scatter_rows": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_vp, _c_vp, _c_i64, _c_vp, _c_i64, _c_i64, _c_vp]),
+    "nvx_moe_glu": (_c_i32, [_c_vp, _c_i32, _c_f32, _c_f32, _c_vp, _c_i64, _c_i64, _c_vp]),
+    "nvx_moe_gather_rows": (_c_i32, [_c_vp, _c_i32, _c_vp, _c_i64, _c_vp, _c_i64, _c_i64, _c_vp]),
 }
 
 _lib = None

@@ -56,9 +56,10 @@ class KVCachePool:
 
 
 class LatentCachePool:
-    """Cache of layers that keep ONE latent vector per token (latent attention): per such layer a tensor
-    (tokens, rank) in the activations' format.  Slot ids are the same token slots the allocator below hands out, so a
-    sequence's slot list serves every layer, whatever its rank."""
+    """Cache of layers that keep rows per token outside the K/V pool: ONE latent vector (latent attention), or a key row and a
+    value row of sizes of their own (attention whose key and value sizes differ from layer to layer).  `ranks`: name ->
+    elements per token; per name a tensor (tokens, rank) in the activations' format.  Slot ids are the same token slots the
+    allocator below hands out, so a sequence's slot list serves every layer, whatever its rank."""
 
     def __init__(self, dtype: torch.dtype, device: torch.device, num_tokens: int, ranks: dict):
         self.dtype, self.device, self.num_tokens = dtype, device, num_tokens

@@ -1,0 +1,180 @@
+// Causal attention over per-token key and value rows addressed through slot lists, for heads whose key size and value size
+// differ, with grouped key/value heads, rotary positions on a leading part of each head (frequencies given as a table, so
+// any scaling of them is the caller's), values scaled to unit mean square before they are cached, and scores that pass
+// cap * tanh(score / cap) before the softmax.
+//   - nvx_rope_vnorm_store: after the fused q|k|v projection: rotate q and k, norm v, scatter k and v into the caches;
+//   - nvx_softcap_attn: the attention itself; scores, maxima, exponentials and sums are float32 in every format.
+#include "fmt_dev.h"
+
+namespace NVX_NS {
+
+// One workgroup per token.  x[t] = [q (heads * dim) | k (kv_heads * dim) | v (kv_heads * vdim)].  The first rot_dims of a
+// head are rotated in pairs (i, i + rot_dims / 2) by the angle positions[t] * freq[i] (the product and its cosine and sine
+// are formed in double precision, so the table alone sets the accuracy), both cos and sin times `mag`.
+template <typename A>
+__global__ __launch_bounds__(256) void rope_vnorm_store_kernel(const A* __restrict__ x, int64_t x_stride, const int64_t* __restrict__ positions,
+                                                              const double* __restrict__ freq, float mag, int rot_dims, float eps,
+                                                              const int64_t* __restrict__ slots, A* __restrict__ q_out,
+                                                              A* __restrict__ k_cache, A* __restrict__ v_cache, int heads, int kv_heads,
+                                                              int dim, int vdim) {
+    extern __shared__ float cs[];      // cos (half), sin (half)
+    const int64_t t = blockIdx.x;
+    const int half = rot_dims / 2;
+    const double pos = (double)positions[t];
+    for (int i = threadIdx.x; i < half; i += 256) {
+        const double a = pos * freq[i];
+        cs[i] = (float)(cos(a) * (double)mag);
+        cs[half + i] = (float)(sin(a) * (double)mag);
+    }
+    __syncthreads();
+    const A* row = x + t * x_stride;
+    const int64_t slot = slots[t];
+    const int nq = heads * dim, nk = kv_heads * dim;
+    for (int idx = threadIdx.x; idx < nq + nk; idx += 256) {
+        const int d = idx % dim;
+        const float v = ld_f(row, idx);
+        float o = v;
+        if (d < half) o = v * cs[d] - ld_f(row, idx + half) * cs[half + d];
+        else if (d < rot_dims) o = v * cs[d - half] + ld_f(row, idx - half) * cs[d];
+        if (idx < nq) st_f(q_out, t * (int64_t)nq + idx, o);
+        else if (slot >= 0) st_f(k_cache, slot * (int64_t)nk + (idx - nq), o);
+    }
+    if (slot < 0) return;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    for (int g = wave; g < kv_heads; g += 4) {
+        const A* v = row + nq + nk + g * vdim;
+        float ss = 0.f;
+        for (int e = lane; e < vdim; e += 64) { const float u = ld_f(v, e); ss += u * u; }
+        const float rn = 1.0f / sqrtf(wave_sum(ss) / (float)vdim + eps);
+        for (int e = lane; e < vdim; e += 64) st_f(v_cache, slot * (int64_t)kv_heads * vdim + g * vdim + e, ld_f(v, e) * rn);
+    }
+}
+
+__device__ __forceinline__ float lane_value(float v, int lane) {      // `lane` is the same in every lane of the wave
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
+// One workgroup of four waves per (head, token).  The waves take the visible keys in tiles of 64, every fourth tile each: a
+// lane scores one key (the query waits in LDS), the wave keeps a running maximum and sum, then each lane accumulates the
+// weighted values of EPL of the head's value columns over the tile's keys.  The four partial results are merged through LDS.
+template <typename A, int EPL>
+__global__ __launch_bounds__(256) void softcap_attn_kernel(const A* __restrict__ q, const A* __restrict__ k_cache, const A* __restrict__ v_cache,
+                                                          const int32_t* __restrict__ kv_indices, const int64_t* __restrict__ kv_start,
+                                                          const int32_t* __restrict__ kv_len, const int32_t* __restrict__ qo_indptr,
+                                                          const int32_t* __restrict__ tok_seq, float scale, float cap, A* __restrict__ out,
+                                                          int heads, int kv_heads, int dim, int vdim) {
+    extern __shared__ float sm[];
+    float* sq = sm;                   // dim
+    float* sacc = sq + dim;           // 4 * vdim
+    float* sml = sacc + 4 * vdim;     // 4 maxima, 4 sums
+    const int hd = blockIdx.x;
+    const int64_t t = blockIdx.y;
+    const int b = tok_seq ? tok_seq[t] : (int)t;
+    const int64_t q0 = qo_indptr ? qo_indptr[b] : b;
+    const int64_t q_n = qo_indptr ? qo_indptr[b + 1] - q0 : 1;
+    const int visible = kv_len[b] - (int)(q_n - 1 - (t - q0));
+    const int kvh = hd / (heads / kv_heads);
+    const int32_t* slots = kv_indices + kv_start[b];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    for (int d = threadIdx.x; d < dim; d += 256) sq[d] = ld_f(q, t * (int64_t)heads * dim + (int64_t)hd * dim + d);
+    __syncthreads();
+    const int64_t k_row = (int64_t)kv_heads * dim, v_row = (int64_t)kv_heads * vdim;
+    float m = -INFINITY, l = 0.f;
+    float acc[EPL];
+#pragma unroll
+    for (int c = 0; c < EPL; ++c) acc[c] = 0.f;
+    for (int j0 = wave * 64; j0 < visible; j0 += 256) {
+        const int j = j0 + lane;
+        const bool valid = j < visible;
+        const int slot = valid ? slots[j] : 0;
+        float s = -INFINITY;
+        if (valid) {
+            const A* kr = k_cache + slot * k_row + (int64_t)kvh * dim;
+            float dot = 0.f;
+            for (int d = 0; d < dim; ++d) dot += sq[d] * ld_f(kr, d);
+            s = dot * scale;
+            if (cap > 0.f) s = cap * tanhf(s / cap);
+        }
+        const float m_new = fmaxf(m, wave_max(s));
+        const float corr = expf(m - m_new);          // first tile: exp(-inf) = 0
+        const float p = valid ? expf(s - m_new) : 0.f;
+        l = l * corr + wave_sum(p);
+        m = m_new;
+#pragma unroll
+        for (int c = 0; c < EPL; ++c) acc[c] *= corr;
+        const int n_here = visible - j0 < 64 ? visible - j0 : 64;
+        for (int jj = 0; jj < n_here; ++jj) {
+            const float pj = lane_value(p, jj);
+            const int sl = __builtin_amdgcn_readlane(slot, jj);
+            const A* vr = v_cache + sl * v_row + (int64_t)kvh * vdim;
+#pragma unroll
+            for (int c = 0; c < EPL; ++c) {
+                const int e = lane + 64 * c;
+                if (e < vdim) acc[c] += pj * ld_f(vr, e);
+            }
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < EPL; ++c) {
+        const int e = lane + 64 * c;
+        if (e < vdim) sacc[wave * vdim + e] = acc[c];
+    }
+    if (lane == 0) { sml[wave] = m; sml[4 + wave] = l; }
+    __syncthreads();
+    const float mm = fmaxf(fmaxf(sml[0], sml[1]), fmaxf(sml[2], sml[3]));
+    float f[4], total = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) { f[w] = expf(sml[w] - mm); total += sml[4 + w] * f[w]; }
+    for (int e = threadIdx.x; e < vdim; e += 256) {
+        float o = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) o += sacc[w * vdim + e] * f[w];
+        st_f(out, t * (int64_t)heads * vdim + (int64_t)hd * vdim + e, o / total);
+    }
+}
+
+}  // namespace NVX_NS
+
+using namespace NVX_NS;
+
+extern "C" int nvx_rope_vnorm_store(const void* x, int64_t x_stride, int fmt, const int64_t* positions, const double* freq, float mag,
+                                    int rot_dims, float eps, const int64_t* slots, void* q_out, void* k_cache, void* v_cache,
+                                    int64_t n_slots, int64_t n_tok, int64_t heads, int64_t kv_heads, int64_t dim, int64_t vdim,
+                                    nvx_stream_t stream) {
+    NVX_REQUIRE(fmt >= 0 && fmt <= 2, NVX_EINVAL, "nvx_rope_vnorm_store: fmt must be 0, 1 or 2");
+    NVX_REQUIRE(n_tok >= 0 && heads > 0 && kv_heads > 0 && dim > 0 && vdim > 0 && n_slots >= 0 && (heads + kv_heads) * dim < (1 << 30) &&
+                    kv_heads * vdim < (1 << 30), NVX_EINVAL, "nvx_rope_vnorm_store: bad sizes");
+    NVX_REQUIRE(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= dim && rot_dims <= 8192, NVX_EINVAL,
+                "nvx_rope_vnorm_store: the rotated part must be even and within a head");
+    NVX_REQUIRE(x_stride >= (heads + kv_heads) * dim + kv_heads * vdim, NVX_EINVAL, "nvx_rope_vnorm_store: row stride");
+    if (n_tok == 0) return NVX_OK;
+    NVX_REQUIRE(x && positions && (freq || rot_dims == 0) && slots && q_out && k_cache && v_cache, NVX_EINVAL, "nvx_rope_vnorm_store: null pointer");
+    NVX_FMT_CALL(fmt, hipLaunchKernelGGL(rope_vnorm_store_kernel<A_>, dim3((unsigned)n_tok), dim3(256), (size_t)(rot_dims + 2) * sizeof(float),
+                                         (hipStream_t)stream, (const A_*)x, x_stride, positions, freq, mag, rot_dims, eps, slots, (A_*)q_out,
+                                         (A_*)k_cache, (A_*)v_cache, (int)heads, (int)kv_heads, (int)dim, (int)vdim));
+    return nvx_check_launch("nvx_rope_vnorm_store");
+}
+
+extern "C" int nvx_softcap_attn(const void* q, const void* k_cache, const void* v_cache, int fmt, const int32_t* kv_indices,
+                                const int64_t* kv_start, const int32_t* kv_len, const int32_t* qo_indptr, const int32_t* tok_seq,
+                                float scale, float cap, void* out, int64_t n_tok, int64_t heads, int64_t kv_heads, int64_t dim, int64_t vdim,
+                                nvx_stream_t stream) {
+    NVX_REQUIRE(fmt >= 0 && fmt <= 2, NVX_EINVAL, "nvx_softcap_attn: fmt must be 0, 1 or 2");
+    NVX_REQUIRE(n_tok >= 0 && n_tok <= 65535 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && dim <= 4096 && vdim > 0 && vdim <= 512,
+                NVX_EINVAL, "nvx_softcap_attn: bad sizes (at most 65535 tokens a step, key size <= 4096, value size <= 512)");
+    if (n_tok == 0) return NVX_OK;
+    NVX_REQUIRE(q && k_cache && v_cache && kv_indices && kv_start && kv_len && out, NVX_EINVAL, "nvx_softcap_attn: null pointer");
+    NVX_REQUIRE((tok_seq != nullptr) == (qo_indptr != nullptr), NVX_EINVAL, "nvx_softcap_attn: tok_seq and qo_indptr go together");
+    const size_t lds = (size_t)(dim + 4 * vdim + 8) * sizeof(float);
+    const dim3 grid((unsigned)heads, (unsigned)n_tok);
+#define NVX_CAP_ATTN(EPL)                                                                                                                 \
+    NVX_FMT_CALL(fmt, hipLaunchKernelGGL((softcap_attn_kernel<A_, EPL>), grid, dim3(256), lds, (hipStream_t)stream, (const A_*)q,          \
+                                         (const A_*)k_cache, (const A_*)v_cache, kv_indices, kv_start, kv_len, qo_indptr, tok_seq, scale,  \
+                                         cap, (A_*)out, (int)heads, (int)kv_heads, (int)dim, (int)vdim))
+    if (vdim <= 64) NVX_CAP_ATTN(1);
+    else if (vdim <= 128) NVX_CAP_ATTN(2);
+    else if (vdim <= 256) NVX_CAP_ATTN(4);
+    else NVX_CAP_ATTN(8);
+#undef NVX_CAP_ATTN
+    return nvx_check_launch("nvx_softcap_attn");
+}

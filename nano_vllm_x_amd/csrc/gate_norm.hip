@@ -1,0 +1,119 @@
+// Sublayer boundaries of stacks whose residual stream is float32, whose norms work on groups of a row, and whose sublayer
+// results pass a learned sigmoid gate before they are added:
+//   - gated residual + grouped RMS norm, one launch per boundary (optionally the result is first formed as the mean of two
+//     RMS-normed branch outputs);
+//   - per-head RMS norm of a recurrence's or attention's read-out, times a weight, times an output gate.
+// Norms, gates and the stream are float32 in every activation format.
+#include "fmt_dev.h"
+
+namespace NVX_NS {
+
+// Per token t (one workgroup):
+//   r = y[t]                                                   (y2 == null)
+//   r = (y[t] / rms(y[t]) * w_y + y2[t] / rms(y2[t]) * w_y2) / 2     (y2 != null; rms over the whole row)
+//   r *= sigmoid(gate[t] + gate_bias)                          (gate != null)
+//   x[t] += mult * r                                           (y != null)
+//   h[t] = x[t], each of `groups` consecutive slices divided by its own root mean square, times w_norm   (w_norm != null)
+template <typename A>
+__global__ __launch_bounds__(256) void gated_residual_norm_kernel(
+    const A* __restrict__ y, int64_t y_stride, const A* __restrict__ y2, int64_t y2_stride, const float* __restrict__ w_y,
+    const float* __restrict__ w_y2, const A* __restrict__ gate, int64_t gate_stride, const float* __restrict__ gate_bias, float mult,
+    float* __restrict__ x, const float* __restrict__ w_norm, int groups, float eps, A* __restrict__ h_out, int width) {
+    __shared__ float red[4];
+    const int64_t t = blockIdx.x;
+    const int64_t row = t * (int64_t)width;
+    const A* yr = y ? y + t * y_stride : nullptr;
+    const A* y2r = y2 ? y2 + t * y2_stride : nullptr;
+    const A* gr = gate ? gate + t * gate_stride : nullptr;
+    float r1 = 1.f, r2 = 1.f;
+    if (y2r) {
+        float a = 0.f, b = 0.f;
+        for (int c = threadIdx.x; c < width; c += 256) {
+            const float u = ld_f(yr, c), v = ld_f(y2r, c);
+            a += u * u;
+            b += v * v;
+        }
+        r1 = 1.0f / sqrtf(block256_sum(a, red) / (float)width + eps);
+        r2 = 1.0f / sqrtf(block256_sum(b, red) / (float)width + eps);
+    }
+    const int gs = width / groups;
+    for (int g = 0; g < groups; ++g) {
+        const int lo = g * gs, hi = lo + gs;
+        float ss = 0.f;
+        for (int c = lo + threadIdx.x; c < hi; c += 256) {
+            float xv = x[row + c];
+            if (yr) {
+                float r = ld_f(yr, c);
+                if (y2r) r = 0.5f * (r * r1 * w_y[c] + ld_f(y2r, c) * r2 * w_y2[c]);
+                if (gr) r *= sigmoid_f(ld_f(gr, c) + (gate_bias ? gate_bias[c] : 0.f));
+                xv += mult * r;
+                x[row + c] = xv;
+            }
+            ss += xv * xv;
+        }
+        if (!w_norm) continue;
+        const float rn = 1.0f / sqrtf(block256_sum(ss, red) / (float)gs + eps);
+        for (int c = lo + threadIdx.x; c < hi; c += 256) st_f(h_out, row + c, x[row + c] * rn * w_norm[c]);   // own stores, read back
+    }
+}
+
+// One wave per (token, head): out = o / rms(o) * w * gate, with gate = 1 (kind 0), sigmoid(z) (1) or z * sigmoid(z) (2) of
+// the gate pre-activations z (same layout as the output).  w has heads * vdim entries, or vdim shared by the heads.
+template <typename A>
+__global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __restrict__ o, const float* __restrict__ w, int w_shared,
+                                                            const A* __restrict__ gate, int64_t gate_stride, int kind, float eps,
+                                                            A* __restrict__ out, int64_t n_rows, int heads, int vdim) {
+    const int64_t idx = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (idx >= n_rows) return;
+    const int lane = threadIdx.x & 63;
+    const int64_t t = idx / heads;
+    const int hd = (int)(idx % heads);
+    const int64_t base = t * (int64_t)heads * vdim + (int64_t)hd * vdim;
+    float ss = 0.f;
+    for (int e = lane; e < vdim; e += 64) { const float v = o[base + e]; ss += v * v; }
+    const float rn = 1.0f / sqrtf(wave_sum(ss) / (float)vdim + eps);
+    for (int e = lane; e < vdim; e += 64) {
+        float v = o[base + e] * rn * w[w_shared ? e : hd * vdim + e];
+        if (kind) {
+            const float z = ld_f(gate, t * gate_stride + (int64_t)hd * vdim + e);
+            v *= kind == 1 ? sigmoid_f(z) : z * sigmoid_f(z);
+        }
+        st_f(out, base + e, v);
+    }
+}
+
+}  // namespace NVX_NS
+
+using namespace NVX_NS;
+
+extern "C" int nvx_gated_residual_norm(const void* y, int64_t y_stride, const void* y2, int64_t y2_stride, const float* w_y,
+                                       const float* w_y2, const void* gate, int64_t gate_stride, const float* gate_bias, int fmt,
+                                       float mult, float* x, const float* w_norm, int groups, float eps, void* h_out, int64_t n_tok,
+                                       int64_t width, nvx_stream_t stream) {
+    NVX_REQUIRE(fmt >= 0 && fmt <= 2, NVX_EINVAL, "nvx_gated_residual_norm: fmt must be 0, 1 or 2");
+    NVX_REQUIRE(n_tok >= 0 && width > 0 && width < (1 << 30) && groups >= 1 && width % groups == 0, NVX_EINVAL,
+                "nvx_gated_residual_norm: bad sizes (the width must be a multiple of the groups)");
+    if (n_tok == 0) return NVX_OK;
+    NVX_REQUIRE(x && (y || w_norm), NVX_EINVAL, "nvx_gated_residual_norm: null pointer");
+    NVX_REQUIRE(!y || y_stride >= width, NVX_EINVAL, "nvx_gated_residual_norm: row stride of y");
+    NVX_REQUIRE(!y2 || (y && w_y && w_y2 && y2_stride >= width), NVX_EINVAL, "nvx_gated_residual_norm: two branches need both weights");
+    NVX_REQUIRE(!gate || (y && gate_stride >= width), NVX_EINVAL, "nvx_gated_residual_norm: a gate needs a result to gate");
+    NVX_REQUIRE(!w_norm || h_out, NVX_EINVAL, "nvx_gated_residual_norm: the norm needs an output");
+    NVX_FMT_CALL(fmt, hipLaunchKernelGGL(gated_residual_norm_kernel<A_>, dim3((unsigned)n_tok), dim3(256), 0, (hipStream_t)stream,
+                                         (const A_*)y, y_stride, (const A_*)y2, y2_stride, w_y, w_y2, (const A_*)gate, gate_stride,
+                                         gate_bias, mult, x, w_norm, groups, eps, (A_*)h_out, (int)width));
+    return nvx_check_launch("nvx_gated_residual_norm");
+}
+
+extern "C" int nvx_head_norm_gate(const float* o, const float* w, int w_shared, const void* gate, int64_t gate_stride, int kind, int fmt,
+                                  float eps, void* out, int64_t n_tok, int64_t heads, int64_t vdim, nvx_stream_t stream) {
+    NVX_REQUIRE(fmt >= 0 && fmt <= 2 && kind >= 0 && kind <= 2, NVX_EINVAL, "nvx_head_norm_gate: fmt must be 0..2, kind 0..2");
+    NVX_REQUIRE(n_tok >= 0 && heads > 0 && vdim > 0 && heads * vdim < (1 << 30), NVX_EINVAL, "nvx_head_norm_gate: bad sizes");
+    if (n_tok == 0) return NVX_OK;
+    NVX_REQUIRE(o && w && out && (kind == 0 || (gate && gate_stride >= heads * vdim)), NVX_EINVAL, "nvx_head_norm_gate: null pointer");
+    const int64_t rows = n_tok * heads;
+    NVX_REQUIRE((rows + 3) / 4 < (1ll << 31), NVX_EINVAL, "nvx_head_norm_gate: too many rows");
+    NVX_FMT_CALL(fmt, hipLaunchKernelGGL(head_norm_gate_kernel<A_>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, (hipStream_t)stream, o, w,
+                                         w_shared, (const A_*)gate, gate_stride, kind, eps, (A_*)out, rows, (int)heads, (int)vdim));
+    return nvx_check_launch("nvx_head_norm_gate");
+}

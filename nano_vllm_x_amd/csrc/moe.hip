@@ -1,0 +1,180 @@
+// Mixture of small gated feed-forward experts with a sigmoid router whose weight scales the chosen expert's INPUT.
+//   - nvx_moe_route: the `top` largest router logits of every token -> expert ids and sigmoid scores (float32);
+//   - nvx_moe_expert_rows: a token's experts evaluated row by row of their weights (a workgroup per token): the form for
+//     steps of few tokens, where every chosen expert's weights have to be streamed once per token anyway;
+//   - nvx_moe_scatter_rows / nvx_moe_glu / nvx_moe_gather_rows: the pieces around per-expert matrix products for steps of
+//     many tokens (scaled inputs gathered into expert order, the gated activation, the tokens' results summed back).
+// Expert:  g = min(W_gate x, limit), u = clamp(W_up x, -limit, limit), y = g sigmoid(alpha g) (u + 1), out = W_down y.
+#include "fmt_dev.h"
+
+namespace NVX_NS {
+
+__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int n_exp, int top, int32_t* __restrict__ idx,
+                                                       float* __restrict__ wts, int64_t n_tok) {
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= n_tok) return;
+    const float* z = logits + t * n_exp;
+    for (int k = 0; k < top; ++k) {
+        int best = -1;
+        float bz = -INFINITY;
+        for (int e = 0; e < n_exp; ++e) {
+            bool taken = false;
+            for (int j = 0; j < k; ++j) taken |= idx[t * top + j] == e;
+            if (!taken && (best < 0 || z[e] > bz)) { best = e; bz = z[e]; }
+        }
+        idx[t * top + k] = best;
+        wts[t * top + k] = sigmoid_f(bz);
+    }
+}
+
+__device__ __forceinline__ float glu_act(float g, float u, float limit, float alpha) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g * sigmoid_f(alpha * g) * (u + 1.0f);
+}
+
+// w_gu: (experts, 2 * ff, width) rows [gate | up]; w_d: (experts, width, ff).  LDS: the scaled input (width), the hidden
+// activations (ff), the running output (width).
+template <typename A>
+__global__ __launch_bounds__(256) void moe_expert_rows_kernel(const A* __restrict__ h, int64_t h_stride, const int32_t* __restrict__ idx,
+                                                             const float* __restrict__ wts, int top, const A* __restrict__ w_gu,
+                                                             const A* __restrict__ w_d, float limit, float alpha, A* __restrict__ out,
+                                                             int width, int ff) {
+    extern __shared__ float sm[];
+    float* xs = sm;
+    float* ys = xs + width;
+    float* os = ys + ff;
+    const int64_t t = blockIdx.x;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    for (int k = 0; k < top; ++k) {
+        const int e = idx[t * top + k];
+        const float wt = wts[t * top + k];
+        __syncthreads();
+        for (int c = threadIdx.x; c < width; c += 256) xs[c] = (float)(A)(wt * ld_f(h, t * h_stride + c));
+        __syncthreads();
+        const A* wg = w_gu + (int64_t)e * 2 * ff * width;
+        for (int j = wave; j < ff; j += 4) {
+            const A* gr = wg + (int64_t)j * width;
+            const A* ur = wg + (int64_t)(ff + j) * width;
+            float g = 0.f, u = 0.f;
+            for (int c = lane; c < width; c += 64) {
+                const float x = xs[c];
+                g += ld_f(gr, c) * x;
+                u += ld_f(ur, c) * x;
+            }
+            g = wave_sum(g);
+            u = wave_sum(u);
+            if (lane == 0) ys[j] = (float)(A)glu_act((float)(A)g, (float)(A)u, limit, alpha);
+        }
+        __syncthreads();
+        const A* wd = w_d + (int64_t)e * width * ff;
+        for (int c = wave; c < width; c += 4) {
+            const A* dr = wd + (int64_t)c * ff;
+            float o = 0.f;
+            for (int j = lane; j < ff; j += 64) o += ld_f(dr, j) * ys[j];
+            o = wave_sum(o);
+            if (lane == 0) os[c] = (k ? os[c] : 0.f) + (float)(A)o;
+        }
+    }
+    __syncthreads();
+    for (int c = threadIdx.x; c < width; c += 256) st_f(out, t * (int64_t)width + c, os[c]);
+}
+
+// xs[dst[r]] = wts[r] * h[r / top]  for every (token, choice) pair r: the experts' inputs in expert order
+template <typename A>
+__global__ __launch_bounds__(256) void moe_scatter_rows_kernel(const A* __restrict__ h, int64_t h_stride, const float* __restrict__ wts,
+                                                              const int64_t* __restrict__ dst, int top, A* __restrict__ xs, int width) {
+    const int64_t r = blockIdx.x;
+    const int64_t t = r / top;
+    const float wt = wts[r];
+    A* o = xs + dst[r] * (int64_t)width;
+    for (int c = threadIdx.x; c < width; c += 256) st_f(o, c, wt * ld_f(h, t * h_stride + c));
+}
+
+// y[r][j] = act(gu[r][j], gu[r][ff + j])
+template <typename A>
+__global__ __launch_bounds__(256) void moe_glu_kernel(const A* __restrict__ gu, A* __restrict__ y, float limit, float alpha, int64_t rows,
+                                                     int ff) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < rows * ff; i += (int64_t)gridDim.x * 256) {
+        const int64_t r = i / ff;
+        const int j = (int)(i % ff);
+        st_f(y, i, glu_act(ld_f(gu, r * 2 * ff + j), ld_f(gu, r * 2 * ff + ff + j), limit, alpha));
+    }
+}
+
+// out[t] = sum_k ys[dst[t * top + k]]
+template <typename A>
+__global__ __launch_bounds__(256) void moe_gather_rows_kernel(const A* __restrict__ ys, const int64_t* __restrict__ dst, int top,
+                                                             A* __restrict__ out, int width) {
+    const int64_t t = blockIdx.x;
+    for (int c = threadIdx.x; c < width; c += 256) {
+        float o = 0.f;
+        for (int k = 0; k < top; ++k) o += ld_f(ys, dst[t * top + k] * (int64_t)width + c);
+        st_f(out, t * (int64_t)width + c, o);
+    }
+}
+
+}  // namespace NVX_NS
+
+using namespace NVX_NS;
+
+extern "C" int nvx_moe_route(const float* logits, int64_t n_tok, int64_t n_exp, int64_t top, int32_t* idx, float* wts, nvx_stream_t stream) {
+    NVX_REQUIRE(n_tok >= 0 && n_exp > 0 && n_exp < (1 << 20) && top > 0 && top <= n_exp, NVX_EINVAL, "nvx_moe_route: bad sizes");
+    if (n_tok == 0) return NVX_OK;
+    NVX_REQUIRE(logits && idx && wts, NVX_EINVAL, "nvx_moe_route: null pointer");
+    hipLaunchKernelGGL(moe_route_kernel, dim3((unsigned)((n_tok + 255) / 256)), dim3(256), 0, (hipStream_t)stream, logits, (int)n_exp, (int)top,
+                       idx, wts, n_tok);
+    return nvx_check_launch("nvx_moe_route");
+}
+
+extern "C" int64_t nvx_moe_expert_rows_max_width(int64_t ff) {
+    const int64_t room = 65536 / 4 - ff;          // floats of the default LDS window left for the input and the output
+    return room > 0 ? room / 2 : 0;
+}
+
+extern "C" int nvx_moe_expert_rows(const void* h, int64_t h_stride, int fmt, const int32_t* idx, const float* wts, int64_t top,
+                                   const void* w_gu, const void* w_d, int64_t n_exp, float limit, float alpha, void* out, int64_t n_tok,
+                                   int64_t width, int64_t ff, nvx_stream_t stream) {
+    NVX_REQUIRE(fmt >= 0 && fmt <= 2, NVX_EINVAL, "nvx_moe_expert_rows: fmt must be 0, 1 or 2");
+    NVX_REQUIRE(n_tok >= 0 && top > 0 && n_exp > 0 && width > 0 && ff > 0 && h_stride >= width, NVX_EINVAL, "nvx_moe_expert_rows: bad sizes");
+    NVX_REQUIRE(width <= nvx_moe_expert_rows_max_width(ff), NVX_EUNSUPPORTED, "nvx_moe_expert_rows: a row and the hidden size do not fit LDS");
+    if (n_tok == 0) return NVX_OK;
+    NVX_REQUIRE(h && idx && wts && w_gu && w_d && out, NVX_EINVAL, "nvx_moe_expert_rows: null pointer");
+    const size_t lds = (size_t)(2 * width + ff) * sizeof(float);
+    NVX_FMT_CALL(fmt, hipLaunchKernelGGL(moe_expert_rows_kernel<A_>, dim3((unsigned)n_tok), dim3(256), lds, (hipStream_t)stream, (const A_*)h,
+                                         h_stride, idx, wts, (int)top, (const A_*)w_gu, (const A_*)w_d, limit, alpha, (A_*)out, (int)width,
+                                         (int)ff));
+    return nvx_check_launch("nvx_moe_expert_rows");
+}
+
+extern "C" int nvx_moe_scatter_rows(const void* h, int64_t h_stride, int fmt, const float* wts, const int64_t* dst, int64_t top, void* xs,
+                                    int64_t n_tok, int64_t width, nvx_stream_t stream) {
+    NVX_REQUIRE(fmt >= 0 && fmt <= 2 && n_tok >= 0 && top > 0 && width > 0 && h_stride >= width && n_tok * top < (1ll << 31), NVX_EINVAL,
+                "nvx_moe_scatter_rows: bad arguments");
+    if (n_tok == 0) return NVX_OK;
+    NVX_REQUIRE(h && wts && dst && xs, NVX_EINVAL, "nvx_moe_scatter_rows: null pointer");
+    NVX_FMT_CALL(fmt, hipLaunchKernelGGL(moe_scatter_rows_kernel<A_>, dim3((unsigned)(n_tok * top)), dim3(256), 0, (hipStream_t)stream,
+                                         (const A_*)h, h_stride, wts, dst, (int)top, (A_*)xs, (int)width));
+    return nvx_check_launch("nvx_moe_scatter_rows");
+}
+
+extern "C" int nvx_moe_glu(const void* gu, int fmt, float limit, float alpha, void* y, int64_t rows, int64_t ff, nvx_stream_t stream) {
+    NVX_REQUIRE(fmt >= 0 && fmt <= 2 && rows >= 0 && ff > 0, NVX_EINVAL, "nvx_moe_glu: bad arguments");
+    if (rows == 0) return NVX_OK;
+    NVX_REQUIRE(gu && y, NVX_EINVAL, "nvx_moe_glu: null pointer");
+    int64_t blocks = (rows * ff + 255) / 256;
+    if (blocks > 256 * 64) blocks = 256 * 64;
+    NVX_FMT_CALL(fmt, hipLaunchKernelGGL(moe_glu_kernel<A_>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const A_*)gu, (A_*)y, limit,
+                                         alpha, rows, (int)ff));
+    return nvx_check_launch("nvx_moe_glu");
+}
+
+extern "C" int nvx_moe_gather_rows(const void* ys, int fmt, const int64_t* dst, int64_t top, void* out, int64_t n_tok, int64_t width,
+                                   nvx_stream_t stream) {
+    NVX_REQUIRE(fmt >= 0 && fmt <= 2 && n_tok >= 0 && n_tok < (1ll << 31) && top > 0 && width > 0, NVX_EINVAL, "nvx_moe_gather_rows: bad arguments");
+    if (n_tok == 0) return NVX_OK;
+    NVX_REQUIRE(ys && dst && out, NVX_EINVAL, "nvx_moe_gather_rows: null pointer");
+    NVX_FMT_CALL(fmt, hipLaunchKernelGGL(moe_gather_rows_kernel<A_>, dim3((unsigned)n_tok), dim3(256), 0, (hipStream_t)stream, (const A_*)ys, dst,
+                                         (int)top, (A_*)out, (int)width));
+    return nvx_check_launch("nvx_moe_gather_rows");
+}

@@ -1,0 +1,58 @@
+"""Mixture of small gated feed-forward experts behind a sigmoid router."""
+from __future__ import annotations
+
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+from .. import ops
+
+
+class SigmoidInputMoE(nn.Module):
+    """scores = sigmoid(W_router h) (float32); every token takes the `top` experts with the largest scores, and a score
+    scales its expert's INPUT (no renormalisation): out = sum_e expert_e(score_e * h).  Expert: g = min(W_gate x, limit),
+    u = clamp(W_up x, -limit, limit), W_down (g * sigmoid(alpha * g) * (u + 1)).
+
+    Steps of few tokens (decode steps, which a hipGraph replays: no host decision may depend on the routing) evaluate each
+    token's experts in one launch, streaming the chosen experts' rows.  Steps of many tokens put the scaled inputs into
+    expert order and run one pair of matrix products per expert that received tokens; the per-expert counts are the one
+    host read of that path."""
+
+    ROWS_PATH_TOKENS = 32
+
+    def __init__(self, width: int, experts: int, top: int, ff: int, limit: float, alpha: float):
+        super().__init__()
+        self.width, self.experts, self.top, self.ff, self.limit, self.alpha = width, experts, top, ff, float(limit), float(alpha)
+        self.router = nn.Parameter(torch.zeros(experts, width, dtype=torch.float32))
+        self.w_gu = nn.Parameter(torch.empty(experts, 2 * ff, width))      # rows of an expert: gate | up
+        self.w_d = nn.Parameter(torch.empty(experts, width, ff))
+        self._rows_fit = None
+
+    def forward(self, h: torch.Tensor, decode_step: bool = False) -> torch.Tensor:
+        t = h.shape[0]
+        idx, wts = ops.moe_route(F.linear(h.float(), self.router), self.top)
+        if self._rows_fit is None:
+            self._rows_fit = ops.moe_expert_rows_fits(self.width, self.ff)
+        if self._rows_fit and (decode_step or t <= self.ROWS_PATH_TOKENS):
+            return ops.moe_expert_rows(h, idx, wts, self.w_gu, self.w_d, self.limit, self.alpha)
+        flat = idx.view(-1).long()
+        order = torch.argsort(flat, stable=True)
+        dst = torch.empty_like(order)
+        dst[order] = torch.arange(order.numel(), device=order.device)
+        dst = dst.view(t, self.top)
+        counts = torch.bincount(flat, minlength=self.experts).tolist()
+        xs = ops.moe_scatter_rows(h, wts, dst)
+        gu = torch.empty((xs.shape[0], 2 * self.ff), dtype=h.dtype, device=h.device)
+        a = 0
+        for e, n in enumerate(counts):
+            if n:
+                torch.mm(xs[a:a + n], self.w_gu[e].t(), out=gu[a:a + n])
+                a += n
+        y = ops.moe_glu(gu, self.limit, self.alpha)
+        ys = torch.empty((xs.shape[0], self.width), dtype=h.dtype, device=h.device)
+        a = 0
+        for e, n in enumerate(counts):
+            if n:
+                torch.mm(y[a:a + n], self.w_d[e].t(), out=ys[a:a + n])
+                a += n
+        return ops.moe_gather_rows(ys, dst)

@@ -39,3 +39,27 @@ class RotaryEmbedding(nn.Module):
         if self.cos_sin_cache.dtype != torch.float32:   # model.to(bf16) casts buffers too
             self.cos_sin_cache = self.cos_sin_cache.float()
         return ops.rope(positions, query, key, self.cos_sin_cache, self.head_size)
+
+
+def rotary_frequencies(dims: int, base: float, scaling: dict | None = None):
+    """(frequencies, magnitude) of a rotation of `dims` dimensions in pairs (i, i + dims / 2): f_i = base^(-2i / dims), float64
+    (dims / 2).  `scaling` = {factor, original, fast, slow} stretches the slow pairs (YaRN: B. Peng, J. Quesnelle, H. Fan,
+    E. Shippole, "YaRN: Efficient Context Window Extension of Large Language Models"): a pair that completes `turns`
+    turns over `original` positions has index d(turns) = dims ln(original / (2 pi turns)) / (2 ln base); between lo =
+    floor(d(fast)) and hi = ceil(d(slow)) (clipped to the table) a ramp goes from 0 to 1, a frequency becomes f / factor
+    where the ramp is 1 and stays f where it is 0, and cos and sin are multiplied by 0.1 ln(factor) + 1."""
+    import math
+
+    idx = torch.arange(dims // 2, dtype=torch.float64)
+    freq = float(base) ** (-2.0 * idx / dims)
+    if not scaling:
+        return freq, 1.0
+    factor, original = float(scaling["factor"]), float(scaling["original"])
+
+    def index_of(turns: float) -> float:
+        return dims * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(float(base)))
+
+    lo = max(math.floor(index_of(float(scaling["fast"]))), 0)
+    hi = min(math.ceil(index_of(float(scaling["slow"]))), dims - 1)
+    ramp = ((idx - lo) / max(hi - lo, 0.001)).clamp_(0.0, 1.0)
+    return freq / factor * ramp + freq * (1.0 - ramp), 0.1 * math.log(factor) + 1.0

@@ -18,8 +18,8 @@ from ..core.kv_cache import LatentCachePool, RecurrentStatePool
 
 
 class SeqStateCache:
-    """`latent_ranks`: layer -> size of the latent it caches per token; `state_shapes`: name -> shape of one sequence's
-    entry (names are the model's: (layer, what))."""
+    """`latent_ranks`: name -> elements a layer caches per token (a latent: the layer's number; keys and values: (layer, "k")
+    and (layer, "v")); `state_shapes`: name -> shape of one sequence's entry (names are the model's: (layer, what))."""
 
     def __init__(self, dtype: torch.dtype, device: torch.device, num_tokens: int, num_slots: int, latent_ranks: dict, state_shapes: dict):
         self.latents = LatentCachePool(dtype, device, num_tokens, latent_ranks)

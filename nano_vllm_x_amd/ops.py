@@ -861,3 +861,281 @@ def latent_attn(q, cache, kv_indices, kv_start, kv_len, layout: StepLayout, scal
     _lib.check(lib.nvx_latent_attn(_ptr(q), _ptr(cache), _fmt(q), _ptr(kv_indices), _ptr(kv_start), _ptr(kv_len), _ptr(layout.qo_indptr),
                                    _ptr(layout.tok_seq), _ptr(gate), _ptr(out), heads, rank, t, float(scale), _stream()), "nvx_latent_attn")
     return out
+
+
+# ---------------------------------------------------------------------------------------------
+# gated residuals with grouped norms, matrix-memory recurrences, capped attention, mixtures of experts
+# ---------------------------------------------------------------------------------------------
+def gated_residual_norm(x, y=None, gate=None, gate_bias=None, mult: float = 1.0, w_norm=None, groups: int = 1, eps: float = 0.0,
+                        y2=None, w_y=None, w_y2=None, dtype=None):
+    """x (T, width) float32, updated in place: x += mult * r with r = y, or the mean of y and y2 after each was divided by its
+    root mean square and multiplied by w_y / w_y2; r passes sigmoid(gate + gate_bias) first if a gate is given.  With
+    `w_norm`, returns the grouped RMS norm of the new x (each of `groups` slices of a row by its own root mean square) times
+    w_norm, in `dtype` (default: y's)."""
+    _dev(x, y, gate, gate_bias, w_norm, y2, w_y, w_y2)
+    _f32c(x, "gated_residual_norm: x")
+    _need(x.dim() == 2, "gated_residual_norm: x must be (T, width)")
+    t, width = x.shape
+    for name, a in (("y", y), ("y2", y2), ("gate", gate)):
+        if a is not None:
+            _need(a.shape == (t, width) and a.stride(1) == 1, f"gated_residual_norm: {name} must be (T, width) with unit inner stride")
+    acts = [a for a in (y, y2, gate) if a is not None]
+    dtype = dtype or (acts[0].dtype if acts else None)
+    _need(dtype in _FMT and all(a.dtype == dtype for a in acts), "gated_residual_norm: y, y2, gate and the output share one format")
+    for name, a in (("gate_bias", gate_bias), ("w_norm", w_norm), ("w_y", w_y), ("w_y2", w_y2)):
+        if a is not None:
+            _f32c(a, "gated_residual_norm: " + name)
+            _need(a.numel() == width, f"gated_residual_norm: {name} size")
+    _need(width % groups == 0, "gated_residual_norm: the width must be a multiple of the groups")
+    h = torch.empty((t, width), dtype=dtype, device=x.device) if w_norm is not None else None
+    lib = _lib.load()
+    _lib.check(lib.nvx_gated_residual_norm(_ptr(y), y.stride(0) if y is not None else 0, _ptr(y2), y2.stride(0) if y2 is not None else 0,
+                                           _ptr(w_y), _ptr(w_y2), _ptr(gate), gate.stride(0) if gate is not None else 0, _ptr(gate_bias),
+                                           _FMT[dtype], float(mult), _ptr(x), _ptr(w_norm), groups, float(eps), _ptr(h), t, width, _stream()),
+               "nvx_gated_residual_norm")
+    return h
+
+
+def head_norm_gate(o, w, eps: float, gate=None, kind: str = "none", dtype=None):
+    """o (T, heads, vdim) float32: every head's row divided by its root mean square, times w ((heads, vdim), or (vdim,) shared
+    by the heads), times the output gate: kind "sigmoid" or "silu" of `gate` (T, heads * vdim).  Returns (T, heads * vdim)."""
+    _dev(o, w, gate)
+    _f32c(o, "head_norm_gate: o")
+    _f32c(w, "head_norm_gate: w")
+    _need(o.dim() == 3, "head_norm_gate: o must be (T, heads, vdim)")
+    t, heads, vdim = o.shape
+    _need(w.numel() in (vdim, heads * vdim), "head_norm_gate: w size")
+    k = {"none": 0, "sigmoid": 1, "silu": 2}[kind]
+    if k:
+        _need(gate is not None and gate.shape == (t, heads * vdim) and gate.stride(1) == 1, "head_norm_gate: gate shape")
+        dtype = dtype or gate.dtype
+        _need(gate.dtype == dtype, "head_norm_gate: gate format")
+    _need(dtype in _FMT, "head_norm_gate: output format")
+    out = torch.empty((t, heads * vdim), dtype=dtype, device=o.device)
+    lib = _lib.load()
+    _lib.check(lib.nvx_head_norm_gate(_ptr(o), _ptr(w), int(w.numel() == vdim), _ptr(gate) if k else None,
+                                      gate.stride(0) if k else 0, k, _FMT[dtype], float(eps), _ptr(out), t, heads, vdim, _stream()),
+               "nvx_head_norm_gate")
+    return out
+
+
+def _layout_args(layout: StepLayout):
+    return _ptr(layout.qo_indptr), _ptr(layout.pos0), _ptr(layout.state_slot)
+
+
+def short_conv_silu(x, w, state, layout: StepLayout):
+    """silu of a causal convolution over time per channel.  x (T, channels) (rows may be a slice of wider rows); w (taps,
+    channels) float32, row j multiplying the input taps - 1 - j tokens back; state (slots, taps - 1, channels) float32, read for
+    the inputs before this step and replaced by each sequence's last ones.  Returns (T, channels) in x's format."""
+    _dev(x, w, state)
+    _need(x.dim() == 2 and x.stride(1) == 1, "short_conv_silu: x must be (T, channels) with unit inner stride")
+    t, ch = x.shape
+    _f32c(w, "short_conv_silu: w")
+    taps = w.shape[0]
+    _need(w.dim() == 2 and w.shape[1] == ch and t == layout.n_tok, "short_conv_silu: shapes")
+    n_slots = 0
+    if taps > 1:
+        _f32c(state, "short_conv_silu: state")
+        _need(state.dim() == 3 and state.shape[1:] == (taps - 1, ch), "short_conv_silu: state shape")
+        n_slots = state.shape[0]
+    out = torch.empty((t, ch), dtype=x.dtype, device=x.device)
+    lib = _lib.load()
+    _lib.check(lib.nvx_short_conv_silu(_ptr(x), x.stride(0), _fmt(x), _ptr(w), taps, _ptr(state) if taps > 1 else None, n_slots,
+                                       _ptr(layout.tok_seq), *_layout_args(layout), _ptr(out), t, layout.n_seq, ch, _stream()),
+               "nvx_short_conv_silu")
+    return out
+
+
+def token_shift_mix(h, mu, state, layout: StepLayout):
+    """out[m] = h + (previous token's h - h) * mu[m].  h (T, width); mu (n_mix, width) float32; state (slots, width) float32:
+    the row before each sequence's first token of this step (zeros at position 0), replaced by its last row.
+    Returns (n_mix, T, width) in h's format."""
+    _dev(h, mu, state)
+    _need(h.dim() == 2 and h.stride(1) == 1, "token_shift_mix: h must be (T, width) with unit inner stride")
+    t, width = h.shape
+    _f32c(mu, "token_shift_mix: mu")
+    _f32c(state, "token_shift_mix: state")
+    _need(mu.dim() == 2 and mu.shape[1] == width and state.dim() == 2 and state.shape[1] == width and t == layout.n_tok, "token_shift_mix: shapes")
+    out = torch.empty((mu.shape[0], t, width), dtype=h.dtype, device=h.device)
+    lib = _lib.load()
+    _lib.check(lib.nvx_token_shift_mix(_ptr(h), h.stride(0), _fmt(h), _ptr(mu), mu.shape[0], _ptr(state), state.shape[0], _ptr(layout.tok_seq),
+                                       *_layout_args(layout), _ptr(out), t, layout.n_seq, width, _stream()), "nvx_token_shift_mix")
+    return out
+
+
+def mlstm_scan(x, offsets, gates, gate_bias, cap: float, mem, norm, peak, layout: StepLayout, heads: int, dim: int, vdim: int):
+    """Matrix memory with a stabilised exponential input gate.  x (T, >= ...): q, k (heads * dim each) and v (heads * vdim) at the
+    three column `offsets`; gates (T, 2 * heads) float32 = input | forget pre-activations, gate_bias (2 * heads); mem (slots,
+    heads, dim, vdim), norm (slots, heads, dim), peak (slots, heads) float32, continued and written back.
+    Returns the read-out (T, heads, vdim) float32."""
+    _dev(x, gates, gate_bias, mem, norm, peak)
+    _need(x.dim() == 2 and x.stride(1) == 1 and x.shape[0] == layout.n_tok, "mlstm_scan: x must be (T, columns) with unit inner stride")
+    t = x.shape[0]
+    for a, what in ((gates, "gates"), (gate_bias, "gate_bias"), (mem, "mem"), (norm, "norm"), (peak, "peak")):
+        _f32c(a, "mlstm_scan: " + what)
+    _need(gates.shape == (t, 2 * heads) and gate_bias.numel() == 2 * heads, "mlstm_scan: gate shapes")
+    n_slots = mem.shape[0]
+    _need(mem.shape == (n_slots, heads, dim, vdim) and norm.shape == (n_slots, heads, dim) and peak.shape == (n_slots, heads), "mlstm_scan: state shapes")
+    out = torch.empty((t, heads, vdim), dtype=F32, device=x.device)
+    lib = _lib.load()
+    _lib.check(lib.nvx_mlstm_scan(_ptr(x), x.stride(0), _fmt(x), offsets[0], offsets[1], offsets[2], _ptr(gates), _ptr(gate_bias), float(cap),
+                                  _ptr(mem), _ptr(norm), _ptr(peak), n_slots, *_layout_args(layout), _ptr(out), t, layout.n_seq, heads, dim, vdim,
+                                  _stream()), "nvx_mlstm_scan")
+    return out
+
+
+def delta_scan(x, offsets, ab, a_log, dt_bias, mem, layout: StepLayout, heads: int, kv_heads: int, dim: int, vdim: int):
+    """Gated delta rule.  x (T, columns): q, k (kv_heads * dim each) and v (heads * vdim) at the three column `offsets`, after
+    their convolution; ab (T, 2 * heads) float32 = decay | write-strength pre-activations; a_log, dt_bias (heads); mem (slots,
+    heads, dim, vdim) float32.  Returns the read-out (T, heads, vdim) float32."""
+    _dev(x, ab, a_log, dt_bias, mem)
+    _need(x.dim() == 2 and x.stride(1) == 1 and x.shape[0] == layout.n_tok, "delta_scan: x must be (T, columns) with unit inner stride")
+    t = x.shape[0]
+    for a, what in ((ab, "ab"), (a_log, "a_log"), (dt_bias, "dt_bias"), (mem, "mem")):
+        _f32c(a, "delta_scan: " + what)
+    _need(ab.shape == (t, 2 * heads) and a_log.numel() == heads and dt_bias.numel() == heads, "delta_scan: gate shapes")
+    n_slots = mem.shape[0]
+    _need(mem.shape == (n_slots, heads, dim, vdim), "delta_scan: state shape")
+    out = torch.empty((t, heads, vdim), dtype=F32, device=x.device)
+    lib = _lib.load()
+    _lib.check(lib.nvx_delta_scan(_ptr(x), x.stride(0), _fmt(x), offsets[0], offsets[1], offsets[2], _ptr(ab), _ptr(a_log), _ptr(dt_bias),
+                                  _ptr(mem), n_slots, *_layout_args(layout), _ptr(out), t, layout.n_seq, heads, kv_heads, dim, vdim, _stream()),
+               "nvx_delta_scan")
+    return out
+
+
+def rwkv_scan(r, k, v, wlog, w0, bonus, mem, layout: StepLayout, heads: int, dim: int):
+    """Decayed outer-product memory read with a bonus for the current token.  r, k, v (T, heads * dim) with one common row
+    stride; wlog (T, heads * dim) float32 and w0 (heads * dim): decay exp(-exp(wlog + w0)); bonus (heads, dim); mem (slots,
+    heads, dim, dim) float32.  Returns the read-out (T, heads, dim) float32."""
+    _dev(r, k, v, wlog, w0, bonus, mem)
+    t = r.shape[0]
+    for a in (r, k, v):
+        _need(a.shape == (t, heads * dim) and a.stride(1) == 1 and a.stride(0) == r.stride(0) and a.dtype == r.dtype, "rwkv_scan: r, k, v shapes")
+    for a, what in ((wlog, "wlog"), (w0, "w0"), (bonus, "bonus"), (mem, "mem")):
+        _f32c(a, "rwkv_scan: " + what)
+    n_slots = mem.shape[0]
+    _need(t == layout.n_tok and wlog.shape == (t, heads * dim) and w0.numel() == heads * dim and bonus.numel() == heads * dim and
+          mem.shape == (n_slots, heads, dim, dim), "rwkv_scan: shapes")
+    out = torch.empty((t, heads, dim), dtype=F32, device=r.device)
+    lib = _lib.load()
+    _lib.check(lib.nvx_rwkv_scan(_ptr(r), _ptr(k), _ptr(v), r.stride(0), _fmt(r), _ptr(wlog), _ptr(w0), _ptr(bonus), _ptr(mem), n_slots,
+                                 *_layout_args(layout), _ptr(out), t, layout.n_seq, heads, dim, _stream()), "nvx_rwkv_scan")
+    return out
+
+
+def rope_vnorm_store(qkv, positions, freq, mag: float, rot_dims: int, eps: float, slots, k_cache, v_cache, heads: int, kv_heads: int,
+                     dim: int, vdim: int):
+    """After the fused projection qkv (T, heads * dim + kv_heads * (dim + vdim)): rotate the first rot_dims of every query and
+    key head by positions * freq (freq: rot_dims / 2 float64; cos and sin times `mag`), divide every value head by its root
+    mean square, store keys and values at k_cache[slots] / v_cache[slots] ((slots, kv_heads * dim) / (slots, kv_heads * vdim), in
+    qkv's format).  Returns the rotated queries (T, heads * dim)."""
+    _dev(qkv, positions, freq, slots, k_cache, v_cache)
+    t = qkv.shape[0]
+    _need(qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] == heads * dim + kv_heads * (dim + vdim), "rope_vnorm_store: qkv shape")
+    _need(positions.dtype == torch.int64 and positions.is_contiguous() and positions.numel() == t, "rope_vnorm_store: positions must be int64 (T)")
+    _need(slots.dtype == torch.int64 and slots.is_contiguous() and slots.numel() == t, "rope_vnorm_store: slots must be int64 (T)")
+    _need(rot_dims == 0 or (freq.dtype == torch.float64 and freq.is_contiguous() and freq.numel() == rot_dims // 2), "rope_vnorm_store: freq must be float64 (rot_dims / 2)")
+    n_slots = k_cache.shape[0]
+    _need(k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype and k_cache.is_contiguous() and v_cache.is_contiguous() and
+          k_cache.shape == (n_slots, kv_heads * dim) and v_cache.shape == (n_slots, kv_heads * vdim), "rope_vnorm_store: cache shapes")
+    q = torch.empty((t, heads * dim), dtype=qkv.dtype, device=qkv.device)
+    lib = _lib.load()
+    _lib.check(lib.nvx_rope_vnorm_store(_ptr(qkv), qkv.stride(0), _fmt(qkv), _ptr(positions), _ptr(freq) if rot_dims else None, float(mag), rot_dims,
+                                        float(eps), _ptr(slots), _ptr(q), _ptr(k_cache), _ptr(v_cache), n_slots, t, heads, kv_heads, dim, vdim,
+                                        _stream()), "nvx_rope_vnorm_store")
+    return q
+
+
+def softcap_attn(q, k_cache, v_cache, kv_indices, kv_start, kv_len, layout: StepLayout, scale: float, cap: float, heads: int,
+                 kv_heads: int, dim: int, vdim: int):
+    """Causal attention of q (T, heads * dim) over cached rows: sequence b's tokens are at slots kv_indices[kv_start[b] :
+    kv_start[b] + kv_len[b]]; scores scale * q . k pass cap * tanh(. / cap) (cap <= 0: not) before the softmax.
+    Returns (T, heads * vdim) in q's format."""
+    _dev(q, k_cache, v_cache, kv_indices, kv_start, kv_len)
+    t = q.shape[0]
+    _need(q.shape == (t, heads * dim) and q.is_contiguous() and t == layout.n_tok, "softcap_attn: q must be contiguous (T, heads * dim)")
+    n_slots = k_cache.shape[0]
+    _need(k_cache.dtype == q.dtype and v_cache.dtype == q.dtype and k_cache.is_contiguous() and v_cache.is_contiguous() and
+          k_cache.shape == (n_slots, kv_heads * dim) and v_cache.shape == (n_slots, kv_heads * vdim), "softcap_attn: cache shapes")
+    _need(kv_indices.dtype == torch.int32 and kv_indices.is_contiguous(), "softcap_attn: kv_indices must be int32")
+    _need(kv_start.dtype == torch.int64 and kv_start.numel() >= layout.n_seq, "softcap_attn: kv_start must be int64 (B)")
+    _need(kv_len.dtype == torch.int32 and kv_len.numel() >= layout.n_seq, "softcap_attn: kv_len must be int32 (B)")
+    out = torch.empty((t, heads * vdim), dtype=q.dtype, device=q.device)
+    lib = _lib.load()
+    _lib.check(lib.nvx_softcap_attn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _fmt(q), _ptr(kv_indices), _ptr(kv_start), _ptr(kv_len),
+                                    _ptr(layout.qo_indptr), _ptr(layout.tok_seq), float(scale), float(cap), _ptr(out), t, heads, kv_heads, dim,
+                                    vdim, _stream()), "nvx_softcap_attn")
+    return out
+
+
+def moe_route(logits, top: int):
+    """logits (T, experts) float32 -> (ids (T, top) int32, scores (T, top) float32): the `top` largest logits of every token
+    (ties: the lower id) and their sigmoids."""
+    _dev(logits)
+    _f32c(logits, "moe_route: logits")
+    t, n_exp = logits.shape
+    idx = torch.empty((t, top), dtype=torch.int32, device=logits.device)
+    wts = torch.empty((t, top), dtype=F32, device=logits.device)
+    lib = _lib.load()
+    _lib.check(lib.nvx_moe_route(_ptr(logits), t, n_exp, top, _ptr(idx), _ptr(wts), _stream()), "nvx_moe_route")
+    return idx, wts
+
+
+def moe_expert_rows_fits(width: int, ff: int) -> bool:
+    return width <= _lib.load().nvx_moe_expert_rows_max_width(ff)
+
+
+def _moe_weights(w_gu, w_d, what: str):
+    n_exp, ff2, width = w_gu.shape
+    _need(w_gu.is_contiguous() and w_d.is_contiguous() and w_d.shape == (n_exp, width, ff2 // 2) and w_d.dtype == w_gu.dtype, what + ": expert weights")
+    return n_exp, ff2 // 2, width
+
+
+def moe_expert_rows(h, idx, wts, w_gu, w_d, limit: float, alpha: float):
+    """out[t] = sum over token t's chosen experts of expert(score * h[t]); w_gu (experts, 2 * ff, width) = gate | up rows, w_d
+    (experts, width, ff).  One workgroup per token: the form for steps of few tokens."""
+    _dev(h, idx, wts, w_gu, w_d)
+    n_exp, ff, width = _moe_weights(w_gu, w_d, "moe_expert_rows")
+    t, top = idx.shape
+    _need(h.shape == (t, width) and h.stride(1) == 1 and h.dtype == w_gu.dtype, "moe_expert_rows: h shape / format")
+    _need(idx.dtype == torch.int32 and idx.is_contiguous() and wts.dtype == F32 and wts.is_contiguous() and wts.shape == idx.shape, "moe_expert_rows: choices")
+    out = torch.empty((t, width), dtype=h.dtype, device=h.device)
+    lib = _lib.load()
+    _lib.check(lib.nvx_moe_expert_rows(_ptr(h), h.stride(0), _fmt(h), _ptr(idx), _ptr(wts), top, _ptr(w_gu), _ptr(w_d), n_exp, float(limit),
+                                       float(alpha), _ptr(out), t, width, ff, _stream()), "nvx_moe_expert_rows")
+    return out
+
+
+def moe_scatter_rows(h, wts, dst):
+    """xs[dst[r]] = wts[r] * h[r // top] for every (token, choice) pair r (dst: int64 (T, top), a permutation)."""
+    _dev(h, wts, dst)
+    t, top = wts.shape
+    _need(h.dim() == 2 and h.shape[0] == t and h.stride(1) == 1 and wts.dtype == F32 and wts.is_contiguous(), "moe_scatter_rows: shapes")
+    _need(dst.dtype == torch.int64 and dst.is_contiguous() and dst.shape == wts.shape, "moe_scatter_rows: dst must be int64 (T, top)")
+    xs = torch.empty((t * top, h.shape[1]), dtype=h.dtype, device=h.device)
+    lib = _lib.load()
+    _lib.check(lib.nvx_moe_scatter_rows(_ptr(h), h.stride(0), _fmt(h), _ptr(wts), _ptr(dst), top, _ptr(xs), t, h.shape[1], _stream()),
+               "nvx_moe_scatter_rows")
+    return xs
+
+
+def moe_glu(gu, limit: float, alpha: float):
+    """gu (rows, 2 * ff) = gate | up pre-activations -> min(g, limit) * sigmoid(alpha * min(g, limit)) * (clamp(u, +-limit) + 1)."""
+    _dev(gu)
+    _need(gu.dim() == 2 and gu.is_contiguous() and gu.shape[1] % 2 == 0, "moe_glu: gu must be contiguous (rows, 2 * ff)")
+    y = torch.empty((gu.shape[0], gu.shape[1] // 2), dtype=gu.dtype, device=gu.device)
+    lib = _lib.load()
+    _lib.check(lib.nvx_moe_glu(_ptr(gu), _fmt(gu), float(limit), float(alpha), _ptr(y), gu.shape[0], gu.shape[1] // 2, _stream()), "nvx_moe_glu")
+    return y
+
+
+def moe_gather_rows(ys, dst):
+    """out[t] = sum_k ys[dst[t][k]]."""
+    _dev(ys, dst)
+    t, top = dst.shape
+    _need(ys.dim() == 2 and ys.is_contiguous() and ys.shape[0] == t * top and dst.dtype == torch.int64 and dst.is_contiguous(), "moe_gather_rows: shapes")
+    out = torch.empty((t, ys.shape[1]), dtype=ys.dtype, device=ys.device)
+    lib = _lib.load()
+    _lib.check(lib.nvx_moe_gather_rows(_ptr(ys), _fmt(ys), _ptr(dst), top, _ptr(out), t, ys.shape[1], _stream()), "nvx_moe_gather_rows")
+    return out

@@ -1,8 +1,8 @@
 """Model registry: config.json names an architecture, the registry gives its configuration reader and model class.
 
 An entry is (read configuration from the parsed config.json, model class).  The model class tells the runner what kind of
-cache it needs through its `family` attribute: "paged_kv" (K and V rows per token: paged attention) or "seq_state" (a
-latent per token and latent layer, plus per-sequence state slots)."""
+cache it needs through its `family` attribute: "paged_kv" (K and V rows per token: paged attention) or "seq_state" (rows
+per token for the layers that attend -- a latent, or keys and values -- plus per-sequence state slots)."""
 from __future__ import annotations
 
 import json
@@ -19,8 +19,13 @@ def _kabidra():
     return KabidraConfig.from_dict, KabidraForCausalLM
 
 
+def _meronex():
+    from .meronex import MeronexConfig, MeronexForCausalLM
+    return MeronexConfig.from_dict, MeronexForCausalLM
+
+
 # architecture name (config.json "architectures"[0] or "architecture") -> loader of (config reader, model class)
-ARCHITECTURES = {"Qwen3ForCausalLM": _qwen3, "Kabidra": _kabidra}
+ARCHITECTURES = {"Qwen3ForCausalLM": _qwen3, "Kabidra": _kabidra, "Meronex": _meronex}
 
 
 def architecture_of(config: dict) -> str:
