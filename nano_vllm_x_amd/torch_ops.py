@@ -68,6 +68,27 @@ _DEFS = {
     "latent_prep": "(Tensor x, Tensor w_q, Tensor w_kv, float eps, Tensor slots, Tensor(a!) cache, int heads) -> (Tensor, Tensor)",
     "latent_attn": "(Tensor q, Tensor cache, Tensor kv_indices, Tensor kv_start, Tensor kv_len, Tensor pos0, Tensor state_slot, "
                    "Tensor? qo_indptr, Tensor? tok_seq, float scale, Tensor? gate) -> Tensor",
+    # gated residuals with grouped norms, matrix-memory recurrences, capped attention, mixtures of experts
+    "gated_residual_norm": "(Tensor(a!) x, Tensor? y, Tensor? gate, Tensor? gate_bias, float mult, Tensor? w_norm, int groups, float eps, "
+                           "Tensor? y2, Tensor? w_y, Tensor? w_y2, ScalarType dtype) -> Tensor?",
+    "head_norm_gate": "(Tensor o, Tensor w, float eps, Tensor? gate, str kind, ScalarType dtype) -> Tensor",
+    "short_conv_silu": "(Tensor x, Tensor w, Tensor(a!)? state, Tensor pos0, Tensor state_slot, Tensor? qo_indptr, Tensor? tok_seq) -> Tensor",
+    "token_shift_mix": "(Tensor h, Tensor mu, Tensor(a!) state, Tensor pos0, Tensor state_slot, Tensor? qo_indptr, Tensor? tok_seq) -> Tensor",
+    "mlstm_scan": "(Tensor x, int q_off, int k_off, int v_off, Tensor gates, Tensor gate_bias, float cap, Tensor(a!) mem, Tensor(b!) norm, "
+                  "Tensor(c!) peak, Tensor pos0, Tensor state_slot, Tensor? qo_indptr, Tensor? tok_seq, int heads, int dim, int vdim) -> Tensor",
+    "delta_scan": "(Tensor x, int q_off, int k_off, int v_off, Tensor ab, Tensor a_log, Tensor dt_bias, Tensor(a!) mem, Tensor pos0, "
+                  "Tensor state_slot, Tensor? qo_indptr, Tensor? tok_seq, int heads, int kv_heads, int dim, int vdim) -> Tensor",
+    "rwkv_scan": "(Tensor r, Tensor k, Tensor v, Tensor wlog, Tensor w0, Tensor bonus, Tensor(a!) mem, Tensor pos0, Tensor state_slot, "
+                 "Tensor? qo_indptr, Tensor? tok_seq, int heads, int dim) -> Tensor",
+    "rope_vnorm_store": "(Tensor qkv, Tensor positions, Tensor? freq, float mag, int rot_dims, float eps, Tensor slots, Tensor(a!) k_cache, "
+                        "Tensor(b!) v_cache, int heads, int kv_heads, int dim, int vdim) -> Tensor",
+    "softcap_attn": "(Tensor q, Tensor k_cache, Tensor v_cache, Tensor kv_indices, Tensor kv_start, Tensor kv_len, Tensor pos0, "
+                    "Tensor state_slot, Tensor? qo_indptr, Tensor? tok_seq, float scale, float cap, int heads, int kv_heads, int dim, int vdim) -> Tensor",
+    "moe_route": "(Tensor logits, int top) -> (Tensor, Tensor)",
+    "moe_expert_rows": "(Tensor h, Tensor idx, Tensor wts, Tensor w_gu, Tensor w_d, float limit, float alpha) -> Tensor",
+    "moe_scatter_rows": "(Tensor h, Tensor wts, Tensor dst) -> Tensor",
+    "moe_glu": "(Tensor gu, float limit, float alpha) -> Tensor",
+    "moe_gather_rows": "(Tensor ys, Tensor dst) -> Tensor",
 }
 for _name, _sig in _DEFS.items():
     _LIB.define(_name + _sig)
@@ -224,6 +245,66 @@ def _latent_prep(x, w_q, w_kv, eps, slots, cache, heads):
 
 def _latent_attn(q, cache, kv_indices, kv_start, kv_len, pos0, state_slot, qo_indptr, tok_seq, scale, gate):
     return ops.latent_attn(q, cache, kv_indices, kv_start, kv_len, _layout(q.shape[1], pos0, state_slot, qo_indptr, tok_seq), scale, gate)
+
+
+def _gated_residual_norm(x, y, gate, gate_bias, mult, w_norm, groups, eps, y2, w_y, w_y2, dtype):
+    return ops.gated_residual_norm(x, y=y, gate=gate, gate_bias=gate_bias, mult=mult, w_norm=w_norm, groups=groups, eps=eps, y2=y2, w_y=w_y,
+                                   w_y2=w_y2, dtype=dtype)
+
+
+def _head_norm_gate(o, w, eps, gate, kind, dtype):
+    return ops.head_norm_gate(o, w, eps, gate=gate, kind=kind, dtype=dtype)
+
+
+def _short_conv_silu(x, w, state, pos0, state_slot, qo_indptr, tok_seq):
+    return ops.short_conv_silu(x, w, state, _layout(x.shape[0], pos0, state_slot, qo_indptr, tok_seq))
+
+
+def _token_shift_mix(h, mu, state, pos0, state_slot, qo_indptr, tok_seq):
+    return ops.token_shift_mix(h, mu, state, _layout(h.shape[0], pos0, state_slot, qo_indptr, tok_seq))
+
+
+def _mlstm_scan(x, q_off, k_off, v_off, gates, gate_bias, cap, mem, norm, peak, pos0, state_slot, qo_indptr, tok_seq, heads, dim, vdim):
+    return ops.mlstm_scan(x, (q_off, k_off, v_off), gates, gate_bias, cap, mem, norm, peak, _layout(x.shape[0], pos0, state_slot, qo_indptr, tok_seq),
+                          heads, dim, vdim)
+
+
+def _delta_scan(x, q_off, k_off, v_off, ab, a_log, dt_bias, mem, pos0, state_slot, qo_indptr, tok_seq, heads, kv_heads, dim, vdim):
+    return ops.delta_scan(x, (q_off, k_off, v_off), ab, a_log, dt_bias, mem, _layout(x.shape[0], pos0, state_slot, qo_indptr, tok_seq), heads,
+                          kv_heads, dim, vdim)
+
+
+def _rwkv_scan(r, k, v, wlog, w0, bonus, mem, pos0, state_slot, qo_indptr, tok_seq, heads, dim):
+    return ops.rwkv_scan(r, k, v, wlog, w0, bonus, mem, _layout(r.shape[0], pos0, state_slot, qo_indptr, tok_seq), heads, dim)
+
+
+def _rope_vnorm_store(qkv, positions, freq, mag, rot_dims, eps, slots, k_cache, v_cache, heads, kv_heads, dim, vdim):
+    return ops.rope_vnorm_store(qkv, positions, freq, mag, rot_dims, eps, slots, k_cache, v_cache, heads, kv_heads, dim, vdim)
+
+
+def _softcap_attn(q, k_cache, v_cache, kv_indices, kv_start, kv_len, pos0, state_slot, qo_indptr, tok_seq, scale, cap, heads, kv_heads, dim, vdim):
+    return ops.softcap_attn(q, k_cache, v_cache, kv_indices, kv_start, kv_len, _layout(q.shape[0], pos0, state_slot, qo_indptr, tok_seq), scale, cap,
+                            heads, kv_heads, dim, vdim)
+
+
+def _moe_route(logits, top):
+    return ops.moe_route(logits, top)
+
+
+def _moe_expert_rows(h, idx, wts, w_gu, w_d, limit, alpha):
+    return ops.moe_expert_rows(h, idx, wts, w_gu, w_d, limit, alpha)
+
+
+def _moe_scatter_rows(h, wts, dst):
+    return ops.moe_scatter_rows(h, wts, dst)
+
+
+def _moe_glu(gu, limit, alpha):
+    return ops.moe_glu(gu, limit, alpha)
+
+
+def _moe_gather_rows(ys, dst):
+    return ops.moe_gather_rows(ys, dst)
 
 
 for _name in _DEFS:

@@ -29,10 +29,6 @@ def grouped_norm(x, w, groups: int, eps: float):
     return rms(parts, eps).reshape(t, width) * w.to(x.dtype)
 
 
-def gelu_tanh(z):
-    return 0.5 * z * (1 + torch.tanh(math.sqrt(2 / math.pi) * (z + 0.044715 * z ** 3)))
-
-
 # ---- rotary positions ----------------------------------------------------------------------------------------------
 def rotary_table(rot: dict, dtype=F64):
     """(frequencies (dims/2), factor on cos and sin) of a rotary specification {base, dims, scaling | None}."""
@@ -56,6 +52,8 @@ def rotary_table(rot: dict, dtype=F64):
 
 def rotate(x, pos, rot: dict):
     """x (T, heads, D); the first rot.dims of D are rotated in pairs (i, i + dims/2) by pos * freq_i."""
+    if not rot:
+        return x
     dims = int(rot["dims"])
     freq, mag = rotary_table(rot, x.dtype)
     ang = pos.to(x.dtype)[:, None] * freq[None, :]
@@ -74,11 +72,12 @@ def softcap_attention(h, p, pre, m: dict, eps: float):
     k = rotate(_lin(p[pre + "k"], h).view(t, g, d), pos, m["rot"])
     v = rms(_lin(p[pre + "v"], h).view(t, g, e), eps)
     out = torch.zeros(t, hq, e, dtype=h.dtype)
-    cap = float(m["softcap"])
+    cap = m.get("softcap")
     for head in range(hq):
         kv = head // (hq // g)
         s = (q[:, head] @ k[:, kv].T) * float(m["scale"])
-        s = cap * torch.tanh(s / cap)
+        if cap:
+            s = float(cap) * torch.tanh(s / float(cap))
         s = s.masked_fill(torch.ones(t, t).triu(1).bool(), float("-inf"))
         out[:, head] = torch.softmax(s, dim=-1) @ v[:, kv]
     return _lin(p[pre + "o"], out.reshape(t, hq * e))

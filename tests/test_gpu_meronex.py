@@ -1,0 +1,547 @@
+"""Meronex through the engine, and its kernels alone, against the plain restatement in oracle/meronex_oracle.py.
+
+Every test makes its own small configuration and weights.  The engine is built on a directory that holds config.json
+(and, where the weights are made by the test, model.safetensors), as a user's would be; steps are given with
+Engine.run_given (the replay entry point) or chosen by the scheduler (Engine.step / LLM.generate).  Comparisons are in
+float32 unless a test says otherwise: there a structural fault (a key too many, a lost state) stands far above rounding.
+"""
+import asyncio
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import meronex_oracle as mo
+
+pytestmark = pytest.mark.gpu
+
+ROT = {"dims": 16, "base": 10000.0, "scaling": {"factor": 4.0, "original": 64, "fast": 16.0, "slow": 1.0}}
+MOE2 = {"kind": "moe", "expert": {"ff": 24, "limit": 2.0}, "router": {"experts": 5, "top": 2}}
+MOE1 = {"kind": "moe", "expert": {"ff": 40, "limit": 0.8}, "router": {"experts": 3, "top": 1}}
+PAR = {"type": "parallel", "mixer": {"left": {"heads": 4, "kv_heads": 2, "dim": 24, "vdim": 40, "rot": ROT, "scale": 0.2, "softcap": 20.0},
+                                     "right": {"heads": 3, "dim": 20, "decay_rank": 5}}, "mlp": MOE2}
+MLS = {"type": "mlstm", "mixer": {"heads": 3, "dim": 20, "vdim": 28, "gate_cap": 8.0}, "mlp": None}
+DEL = {"type": "delta", "mixer": {"heads": 4, "kv_heads": 2, "dim": 40, "vdim": 24, "conv": 4}, "mlp": MOE1}
+
+
+def make_cfg(layers, width=48, vocab=67, groups=3, eps=1e-5, mult=0.7):
+    return {"architecture": "Meronex", "vocab": vocab, "width": width, "norm": {"eps": eps, "groups": groups}, "residual_mult": mult,
+            "layers": json.loads(json.dumps(layers))}
+
+
+def model_dir(tmp_path, cfg, weights=None, name="m"):
+    d = tmp_path / name
+    d.mkdir()
+    (d / "config.json").write_text(json.dumps(cfg))
+    if weights is not None:
+        from safetensors.torch import save_file
+        save_file({k: v.to(torch.bfloat16).contiguous() for k, v in weights.items()}, str(d / "model.safetensors"))
+    return str(d)
+
+
+def weights_of(cfg, seed=0):
+    """The weights an engine built on a directory without a checkpoint draws for `seed`."""
+    from nano_vllm_x_amd.meronex import MeronexConfig, random_checkpoint
+    return dict(random_checkpoint(MeronexConfig.from_dict(cfg), seed))
+
+
+def make_engine(path, dtype="float32", pool=2048, max_bs=4, seed=0, **kw):
+    from nano_vllm_x_amd.core.engine import Engine
+    return Engine(model=path, gpu_memory_utilization=0.5, max_bs=max_bs, enforce_eager=True, context_len=pool, kv_cache_size=pool,
+                  dtype=dtype, seed=seed, **kw)
+
+
+def replay(engine, requests, schedule):
+    """requests: id -> tokens; schedule: list of steps, each a list of (id, n).  Logits of every token, id -> (T, vocab)."""
+    from nano_vllm_x_amd.core.common import SamplingParams
+    at = {i: 0 for i in requests}
+    rows = {i: [] for i in requests}
+    for step in schedule:
+        plan, want = [], []
+        for i, n in step:
+            piece = list(requests[i][at[i]:at[i] + n])
+            if engine.scheduler.get_sequence(i) is None:
+                engine.add_sequence(i, piece, SamplingParams(ignore_eos=True))
+            else:
+                engine.extend_sequence(i, piece)
+            plan.append((i, n))
+            want.append(list(range(n)))
+        out = engine.run_given(plan, want).float().cpu()
+        k = 0
+        for i, n in step:
+            rows[i].append(out[k:k + n])
+            k += n
+            at[i] += n
+            if at[i] == len(requests[i]):
+                engine.abort_sequence(i)
+    return {i: torch.cat(r) for i, r in rows.items()}
+
+
+def close(got, want, tol, what=""):
+    got, want = got.double(), want.double()
+    scale = want.std().item() + 1e-12
+    err = (got - want).abs().max().item() / scale
+    assert err < tol, f"{what}: max error {err:.3e} of the values' spread (tolerance {tol})"
+
+
+def tokens(n, vocab, seed):
+    return torch.randint(0, vocab, (n,), generator=torch.Generator().manual_seed(seed)).tolist()
+
+
+def cuts_of(n, sizes):
+    """n tokens cut into portions whose sizes cycle through `sizes`."""
+    out, k = [], 0
+    while n > 0:
+        c = min(sizes[k % len(sizes)], n)
+        out.append(c)
+        n -= c
+        k += 1
+    return out
+
+
+F32_TOL = 2e-4
+
+
+def _layout(ops, lens, pos0, slots, decode=False):
+    n = len(lens)
+    p, s = torch.tensor(pos0, dtype=torch.int64).cuda(), torch.tensor(slots, dtype=torch.int32).cuda()
+    if decode:
+        return ops.StepLayout(n, n, p, s)
+    qo = np.zeros(n + 1, dtype=np.int32)
+    np.cumsum(lens, out=qo[1:])
+    tok = np.repeat(np.arange(n, dtype=np.int32), lens)
+    return ops.StepLayout(int(qo[-1]), n, p, s, torch.from_numpy(qo).cuda(), torch.from_numpy(tok).cuda())
+
+
+# ---- kernels alone -------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("fmt", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("groups", [1, 2, 5])
+def test_gated_residual_and_grouped_norm(fmt, groups):
+    from nano_vllm_x_amd import ops
+    g = torch.Generator().manual_seed(groups)
+    t, w = 6, 70 * groups          # slices of 70: no vector width divides them
+    x = torch.randn(t, w, generator=g)
+    y, y2, gate = (torch.randn(t, w, generator=g).to(fmt) for _ in range(3))
+    bias, wn, wy, wy2 = (torch.randn(w, generator=g) for _ in range(4))
+    tol = 1e-5 if fmt == torch.float32 else 2e-2
+    # norm alone
+    xd = x.cuda()
+    h = ops.gated_residual_norm(xd, w_norm=wn.cuda(), groups=groups, eps=1e-3, dtype=fmt)
+    assert torch.equal(xd.cpu(), x) and torch.allclose(h.float().cpu(), mo.grouped_norm(x, wn, groups, 1e-3), atol=tol)
+    # one branch, gated
+    xd = x.cuda()
+    h = ops.gated_residual_norm(xd, y=y.cuda(), gate=gate.cuda(), gate_bias=bias.cuda(), mult=0.3, w_norm=wn.cuda(), groups=groups, eps=1e-3)
+    want = x + 0.3 * y.float() * torch.sigmoid(gate.float() + bias)
+    assert torch.allclose(xd.cpu(), want, atol=1e-5) and torch.allclose(h.float().cpu(), mo.grouped_norm(want, wn, groups, 1e-3), atol=tol)
+    # the mean of two normed branches, no norm after
+    xd = x.cuda()
+    assert ops.gated_residual_norm(xd, y=y.cuda(), y2=y2.cuda(), w_y=wy.cuda(), w_y2=wy2.cuda(), gate=gate.cuda(), mult=2.0, eps=1e-3) is None
+    r = 0.5 * (mo.rms(y.float(), 1e-3) * wy + mo.rms(y2.float(), 1e-3) * wy2)
+    assert torch.allclose(xd.cpu(), x + 2.0 * r * torch.sigmoid(gate.float()), atol=1e-5)
+
+
+@pytest.mark.parametrize("kind", ["none", "sigmoid", "silu"])
+@pytest.mark.parametrize("shared", [False, True])
+def test_head_norm_and_output_gate(kind, shared):
+    from nano_vllm_x_amd import ops
+    g = torch.Generator().manual_seed(3)
+    t, heads, vdim = 5, 3, 70
+    o = torch.randn(t, heads, vdim, generator=g)
+    w = torch.randn(vdim if shared else heads * vdim, generator=g)
+    z = torch.randn(t, heads * vdim, generator=g)
+    got = ops.head_norm_gate(o.cuda(), w.cuda(), 1e-4, gate=z.cuda() if kind != "none" else None, kind=kind, dtype=torch.float32)
+    want = mo.rms(o, 1e-4) * (w if shared else w.view(heads, vdim))
+    want = want.reshape(t, -1) * {"none": 1.0, "sigmoid": torch.sigmoid(z), "silu": z * torch.sigmoid(z)}[kind]
+    assert torch.allclose(got.cpu(), want, atol=1e-5)
+
+
+@pytest.mark.parametrize("taps", [1, 2, 3, 6])
+def test_short_convolution_continues_over_cuts_and_reused_slots(taps):
+    """Two sequences in slots that are not in order, cut into steps of 1, 2, taps - 1, taps and more tokens; a third
+    sequence later takes over a used slot and must not see what is left there."""
+    from nano_vllm_x_amd import ops
+    g = torch.Generator().manual_seed(taps)
+    ch = 70
+    k = torch.randn(ch, taps, generator=g)
+    full = {0: torch.randn(23, ch, generator=g), 1: torch.randn(17, ch, generator=g), 2: torch.randn(9, ch, generator=g)}
+    want = {i: mo.short_conv_silu(h, k) for i, h in full.items()}
+    state = torch.full((3, taps - 1, ch), 7.0).cuda() if taps > 1 else None
+    slot = {0: 2, 1: 0, 2: 2}
+    cuts = {0: cuts_of(23, [1, 2, max(taps - 1, 1), taps, 1, 1, 23]), 1: cuts_of(17, [5, 1, 1, 2, 17]), 2: cuts_of(9, [2, 1, 6])}
+    at = {0: 0, 1: 0, 2: 0}
+    got = {i: [] for i in full}
+    kw = k.t().contiguous().cuda()
+    order = [[0, 1]] * 4 + [[0]] * 10 + [[1]] * 5 + [[2, 1]] * 5     # sequence 2 starts in slot 2 after sequence 0 is done
+    for live in order:
+        live = [i for i in live if at[i] < len(full[i]) and cuts[i]]
+        if not live:
+            continue
+        lens = [cuts[i].pop(0) for i in live]
+        x = torch.cat([full[i][at[i]:at[i] + n] for i, n in zip(live, lens)]).cuda()
+        decode = all(n == 1 for n in lens) and all(at[i] > 0 for i in live)
+        out = ops.short_conv_silu(x, kw, state, _layout(ops, lens, [at[i] for i in live], [slot[i] for i in live], decode)).cpu()
+        a = 0
+        for i, n in zip(live, lens):
+            got[i].append(out[a:a + n])
+            a += n
+            at[i] += n
+    for i in full:
+        assert at[i] == len(full[i])
+        assert torch.allclose(torch.cat(got[i]), want[i], atol=1e-5), i
+
+
+def test_token_shift_reads_the_row_before_each_portion():
+    from nano_vllm_x_amd import ops
+    g = torch.Generator().manual_seed(5)
+    w = 50
+    mu = torch.rand(5, w, generator=g)
+    h = torch.randn(14, w, generator=g)
+    prev = torch.cat([torch.zeros(1, w), h[:-1]])
+    want = h[None] + (prev - h)[None] * mu[:, None]
+    state = torch.full((2, w), 9.0).cuda()
+    got, at = [], 0
+    for n in [1, 1, 2, 5, 1, 4]:
+        lay = _layout(ops, [n], [at], [1], decode=(n == 1 and at > 0))
+        got.append(ops.token_shift_mix(h[at:at + n].cuda(), mu.cuda(), state, lay).cpu())
+        at += n
+    assert torch.allclose(torch.cat(got, dim=1), want, atol=1e-6)
+    assert torch.equal(state[0].cpu(), torch.full((w,), 9.0))
+
+
+def test_rotation_with_stretched_frequencies():
+    """Frequencies and magnitude of the product against the restatement's, for a table whose ramp starts inside it and one
+    that has no scaling; then the rotation kernel at positions up to several thousand."""
+    from nano_vllm_x_amd import ops
+    from nano_vllm_x_amd.layers.rotary_embedding import rotary_frequencies
+    for rot in (ROT, {"dims": 8, "base": 500.0, "scaling": None}, {"dims": 32, "base": 1e6, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 2.0}}):
+        f, mag = rotary_frequencies(rot["dims"], rot["base"], rot["scaling"])
+        f2, mag2 = mo.rotary_table(rot)
+        assert torch.allclose(f, f2, rtol=1e-12) and abs(mag - mag2) < 1e-12
+    g = torch.Generator().manual_seed(2)
+    heads, kvh, dim, vdim, t = 3, 1, 24, 10, 6
+    x = torch.randn(t, heads * dim + kvh * (dim + vdim), generator=g)
+    pos = torch.tensor([0, 1, 63, 64, 999, 5000])
+    slots = torch.tensor([4, 0, -1, 2, 5, 1])
+    kc, vc = torch.zeros(6, kvh * dim).cuda(), torch.zeros(6, kvh * vdim).cuda()
+    f, mag = rotary_frequencies(ROT["dims"], ROT["base"], ROT["scaling"])
+    q = ops.rope_vnorm_store(x.cuda(), pos.cuda(), f.cuda(), mag, ROT["dims"], 1e-5, slots.cuda(), kc, vc, heads, kvh, dim, vdim).cpu()
+    x64 = x.double()
+    want_q = mo.rotate(x64[:, :heads * dim].view(t, heads, dim), pos, ROT).reshape(t, -1)
+    want_k = mo.rotate(x64[:, heads * dim:(heads + kvh) * dim].view(t, kvh, dim), pos, ROT).reshape(t, -1)
+    want_v = mo.rms(x64[:, (heads + kvh) * dim:].view(t, kvh, vdim), 1e-5).reshape(t, -1)
+    assert torch.allclose(q.double(), want_q, atol=2e-6)
+    keep = slots >= 0
+    assert torch.allclose(kc.cpu().double()[slots[keep]], want_k[keep], atol=2e-6)
+    assert torch.allclose(vc.cpu().double()[slots[keep]], want_v[keep], atol=2e-6)
+    assert torch.equal(kc.cpu()[3], torch.zeros(kvh * dim))        # the token with a negative slot stored nothing
+
+
+@pytest.mark.parametrize("fmt", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("vdim", [10, 100, 200, 300])
+def test_capped_attention_finds_one_key_among_hundreds(fmt, vdim):
+    """Keys scattered over the pool in a shuffled order; one key far back carries a score that stands out only through the
+    cap's shape (its raw score is far above the cap, the others' are small), so the read-out is that key's value unless a
+    key is lost, the mask is off by one, or the cap is left out.  The last query sees itself; the one before must not see it."""
+    from nano_vllm_x_amd import ops
+    g = torch.Generator().manual_seed(vdim)
+    heads, kvh, dim, n, pool, cap, scale = 4, 2, 24, 700, 1024, 6.0, 0.5
+    k = 0.05 * torch.randn(n, kvh, dim, generator=g)
+    v = torch.randn(n, kvh, vdim, generator=g)
+    q = torch.randn(3, heads, dim, generator=g)          # queries of the last three tokens
+    needle = 37
+    k[needle, 0] = q[1, 1] / q[1, 1].norm() * 40.0       # head 1 (key/value head 0) of the middle query points at it
+    k[n - 1, 1] = q[2, 3] / q[2, 3].norm() * 40.0        # head 3 of the last query points at the last key: itself
+    slots = torch.randperm(pool, generator=g)[:n].to(torch.int32)
+    kc, vc = torch.zeros(pool, kvh * dim, dtype=fmt), torch.zeros(pool, kvh * vdim, dtype=fmt)
+    kc[slots.long()], vc[slots.long()] = k.view(n, -1).to(fmt), v.view(n, -1).to(fmt)
+    lay = _layout(ops, [3], [n - 3], [0])
+    out = ops.softcap_attn(q.view(3, -1).to(fmt).cuda(), kc.cuda(), vc.cuda(), slots.cuda(), torch.tensor([0]).cuda(),
+                           torch.tensor([n], dtype=torch.int32).cuda(), lay, scale, cap, heads, kvh, dim, vdim).float().cpu().view(3, heads, vdim)
+    kf, vf, qf = k.to(fmt).double(), v.to(fmt).double(), q.to(fmt).double()
+    for i in range(3):
+        vis = n - 2 + i
+        for h in range(heads):
+            s = cap * torch.tanh((kf[:vis, h // 2] @ qf[i, h]) * scale / cap)
+            want = torch.softmax(s, 0) @ vf[:vis, h // 2]
+            assert torch.allclose(out[i, h].double(), want, atol=1e-5 if fmt == torch.float32 else 2e-2), (i, h)
+    # the needle's weight: e^(cap) against about n keys at e^(~0): it dominates, and an uncapped score would make it the only key
+    s = cap * torch.tanh((kf[:n - 1, 0] @ qf[1, 1]) * scale / cap)
+    p = torch.softmax(s, 0)
+    assert 0.2 < p[needle] < 0.9
+    assert (out[1, 3] - out[2, 3]).abs().max() > 0.1          # the last query's own key changes head 3
+
+
+@pytest.mark.parametrize("top,experts", [(1, 1), (1, 4), (2, 5), (3, 3)])
+def test_experts_by_rows_and_by_expert_order_agree_with_the_restatement(top, experts):
+    from nano_vllm_x_amd.layers.moe import SigmoidInputMoE
+    g = torch.Generator().manual_seed(10 * top + experts)
+    w, ff, limit, t = 50, 30, 0.7, 45
+    p = {"router": torch.randn(experts, w, generator=g)}
+    for e in range(experts):
+        p.update({f"e{e}.gate": torch.randn(ff, w, generator=g) * 0.3, f"e{e}.up": torch.randn(ff, w, generator=g) * 0.3,
+                  f"e{e}.down": torch.randn(w, ff, generator=g) * 0.2})
+    h = torch.randn(t, w, generator=g)
+    spec = {"expert": {"ff": ff, "limit": limit}, "router": {"experts": experts, "top": top}}
+    want = mo.moe(h.double(), {k: v.double() for k, v in p.items()}, "", spec)
+    moe = SigmoidInputMoE(w, experts, top, ff, limit, 1.702).to(torch.float32).cuda()
+    with torch.no_grad():
+        moe.router.copy_(p["router"])
+        for e in range(experts):
+            moe.w_gu[e, :ff].copy_(p[f"e{e}.gate"])
+            moe.w_gu[e, ff:].copy_(p[f"e{e}.up"])
+            moe.w_d[e].copy_(p[f"e{e}.down"])
+        by_expert = moe(h.cuda()).cpu()                      # 45 tokens: per-expert matrix products
+        by_rows = moe(h.cuda(), decode_step=True).cpu()      # the same tokens as a decode step would take them
+    close(by_expert, want, 1e-5, "by expert")
+    close(by_rows, want, 1e-5, "by rows")
+    assert (want.abs() > 0).all()
+
+
+# ---- one mixer at a time through the engine, over cuts --------------------------------------------------------------------
+ONE = {"mlstm": [MLS], "delta": [DEL], "parallel": [PAR],
+       "mlstm, wide key": [{"type": "mlstm", "mixer": {"heads": 2, "dim": 72, "vdim": 136, "gate_cap": 15.0}, "mlp": MOE1}],
+       "delta, one tap, no groups": [{"type": "delta", "mixer": {"heads": 2, "kv_heads": 2, "dim": 33, "vdim": 70, "conv": 1}, "mlp": None}],
+       "parallel, one head each": [{"type": "parallel", "mlp": None, "mixer": {
+           "left": {"heads": 1, "kv_heads": 1, "dim": 8, "vdim": 8, "rot": {"dims": 8, "base": 100.0, "scaling": None}, "scale": 1.0, "softcap": None},
+           "right": {"heads": 1, "dim": 48, "decay_rank": 1}}}]}
+
+
+@pytest.mark.parametrize("name", list(ONE))
+def test_each_mixer_alone_whole_cut_and_token_by_token(tmp_path, name):
+    cfg = make_cfg(ONE[name], groups=1 if "no groups" in name else 3)
+    w = weights_of(cfg, 1)
+    eng = make_engine(model_dir(tmp_path, cfg, w), pool=256)
+    toks = tokens(61, cfg["vocab"], 3)
+    want = mo.forward(cfg, w, toks)
+    close(replay(eng, {"a": toks}, [[("a", 61)]])["a"], want, F32_TOL, "whole")
+    close(replay(eng, {"b": toks}, [[("b", n)] for n in cuts_of(61, [2, 7, 1, 9, 3, 8, 16])])["b"], want, F32_TOL, "cut")
+    close(replay(eng, {"c": toks}, [[("c", 1)]] * 61)["c"], want, F32_TOL, "token by token")
+    eng.shutdown()
+
+
+# ---- the whole stack ------------------------------------------------------------------------------------------------------
+def test_batches_of_unequal_requests_in_a_small_pool(tmp_path):
+    """Four live requests at most in a pool smaller than the sum of all: portions beside single tokens, a request that
+    pauses for some steps, slots and state slots that change hands (six requests, four state slots)."""
+    cfg = make_cfg([PAR, MLS, DEL, PAR])
+    w = weights_of(cfg, 2)
+    eng = make_engine(model_dir(tmp_path, cfg, w), pool=160, max_bs=4)
+    req = {f"r{k}": tokens(n, cfg["vocab"], 30 + k) for k, n in enumerate([70, 41, 1, 23, 55, 38])}
+    want = {i: mo.forward(cfg, w, t) for i, t in req.items()}
+    sched = [[("r0", 16), ("r1", 2)], [("r0", 1), ("r1", 30), ("r2", 1)], [("r0", 40), ("r3", 3)], [("r1", 1), ("r3", 1)],
+             [("r0", 1), ("r1", 1), ("r3", 17)], [("r0", 12), ("r1", 7), ("r3", 2)],          # r0, r1, r3 done: 134 slots come back
+             [("r4", 2), ("r5", 30)], [("r4", 50), ("r5", 1)], [("r4", 1), ("r5", 1)], [("r4", 2), ("r5", 6)]]
+    got = replay(eng, req, sched)
+    for i in req:
+        close(got[i], want[i], F32_TOL, i)
+    assert eng.scheduler.state_slots.num_free() == 4
+    eng.shutdown()
+
+
+def _sharpened(cfg, seed):
+    """Weights that make far tokens count: attention queries and keys scaled up (peaked scores), forget gates and decays
+    pushed towards keeping (old state survives hundreds of tokens)."""
+    w = weights_of(cfg, seed)
+    for name in w:
+        if name.endswith(("left.q", "left.k")):
+            w[name] = w[name] * 3.0
+        if name.endswith(".f.b"):
+            w[name] = w[name] + 3.0
+        if name.endswith((".A_log", ".w0")):
+            w[name] = w[name] - 3.0
+    return {k: v.to(torch.bfloat16).float() for k, v in w.items()}
+
+
+def test_far_tokens_and_old_state_count(tmp_path):
+    cfg = make_cfg([PAR, DEL, MLS, PAR])
+    w = _sharpened(cfg, 7)
+    eng = make_engine(model_dir(tmp_path, cfg, w), pool=512)
+    toks = tokens(330, cfg["vocab"], 2)
+    want = mo.forward(cfg, w, toks)
+    got = replay(eng, {"a": toks}, [[("a", 255)], [("a", 1)], [("a", 1)], [("a", 2)], [("a", 30)]] + [[("a", 1)]] * 41)["a"]
+    close(got, want, F32_TOL, "sharpened")
+    # the same prompt without its first token is another function of the rest: the first token is seen at the end
+    other = mo.forward(cfg, w, toks[1:])
+    assert (other[-1] - want[-1]).abs().max() > 20 * F32_TOL * want.std()
+    eng.shutdown()
+
+
+def test_bfloat16_stays_within_rounding(tmp_path):
+    cfg = make_cfg([PAR, MLS, DEL])
+    toks = tokens(90, cfg["vocab"], 4)
+    want = mo.forward(cfg, weights_of(cfg, 2), toks)
+    eng = make_engine(model_dir(tmp_path, cfg), dtype="bfloat16", seed=2)
+    got = replay(eng, {"a": toks}, [[("a", 50)], [("a", 2)]] + [[("a", 1)]] * 38)["a"]
+    # a token whose two best experts are a rounding apart may take the other one: judge the bulk, bound the worst
+    err = (got.double() - want).abs().amax(dim=1) / want.std()
+    assert err.median() < 0.08 and err.max() < 0.6, (err.median().item(), err.max().item())
+    eng.shutdown()
+
+
+def test_checkpoint_with_a_missing_or_misshapen_tensor_is_refused(tmp_path):
+    cfg = make_cfg([PAR])
+    w = weights_of(cfg, 0)
+    bad = dict(w)
+    del bad["l0.mix.right.mu.g"]
+    with pytest.raises(KeyError):
+        make_engine(model_dir(tmp_path, cfg, bad, name="missing"))
+    bad = dict(w)
+    bad["l0.mix.left.v"] = torch.zeros(81, cfg["width"])
+    with pytest.raises(ValueError):
+        make_engine(model_dir(tmp_path, cfg, bad, name="shape"))
+    # the decay's inner size comes with the checkpoint: another one loads, and computes with it
+    rank = dict(w)
+    g = torch.Generator().manual_seed(1)
+    rank["l0.mix.right.w1"] = (torch.randn(9, cfg["width"], generator=g) * 0.2).to(torch.bfloat16).float()
+    rank["l0.mix.right.w2"] = (torch.randn(60, 9, generator=g) * 0.3).to(torch.bfloat16).float()
+    eng = make_engine(model_dir(tmp_path, cfg, rank, name="rank"), pool=64)
+    toks = tokens(20, cfg["vocab"], 1)
+    close(replay(eng, {"a": toks}, [[("a", 20)]])["a"], mo.forward(cfg, rank, toks), F32_TOL, "another decay rank")
+    eng.shutdown()
+
+
+# ---- generation: the scheduler's own choices ---------------------------------------------------------------------------
+def oracle_greedy(w, cfg, prompt, n_new):
+    toks = list(prompt)
+    for _ in range(n_new):
+        toks.append(int(mo.forward(cfg, w, toks)[-1].argmax()))
+    return toks[len(prompt):]
+
+
+@pytest.mark.parametrize("chunked", [False, True], ids=["whole prompts", "chunked prefill"])
+def test_greedy_generation_through_the_engine(tmp_path, chunked):
+    """Prompts of unequal length admitted together, decoded as one batch; more requests than state slots, so the later
+    ones wait for a slot that an earlier one gives back; with chunked prefill the prompts are computed in portions of
+    seven tokens.  Long decoding (30 tokens) for one of them."""
+    from nano_vllm_x_amd.core.common import SamplingParams
+    cfg = make_cfg([PAR, MLS, DEL])
+    kw = dict(max_prefill_tokens=7, chunked_prefill=True) if chunked else {}
+    eng = make_engine(model_dir(tmp_path, cfg), pool=300, max_bs=3, seed=9, **kw)
+    w = weights_of(cfg, 9)
+    prompts = {f"r{k}": tokens(n, cfg["vocab"], 20 + k) for k, n in enumerate([5, 19, 1, 12, 9])}
+    new = {"r0": 30, "r1": 5, "r2": 8, "r3": 4, "r4": 6}
+    for i, p in prompts.items():
+        eng.add_sequence(i, list(p), SamplingParams(temperature=0.0, ignore_eos=True, max_new_tokens=new[i]))
+    out = {i: [] for i in prompts}
+    steps = 0
+    while eng.has_unfinished_sequences():
+        for o in eng.step():
+            out[o.seq_id].append(o.new_token_id)
+        steps += 1
+        assert steps < 400
+    for i, p in prompts.items():
+        assert out[i] == oracle_greedy(w, cfg, p, new[i]), i
+    assert eng.scheduler.state_slots.num_free() == 3
+    eng.shutdown()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_steps_replay_a_captured_graph(tmp_path, dtype):
+    """With graphs on, every decode step replays the graph of its batch size, with prefill steps of later requests (eager
+    work on the same cache and state) between the replays; batch sizes change as requests end.  float32: the tokens are
+    the restatement's; bfloat16: the graph's tokens are those of eager steps (same kernels, same order)."""
+    from nano_vllm_x_amd.core.common import SamplingParams
+    from nano_vllm_x_amd.core.engine import Engine
+    cfg = make_cfg([PAR, MLS, DEL, PAR])
+    path = model_dir(tmp_path, cfg)
+    prompts = {f"r{k}": tokens(n, cfg["vocab"], 40 + k) for k, n in enumerate([9, 26, 2, 17, 5])}
+    new = {"r0": 20, "r1": 5, "r2": 11, "r3": 3, "r4": 7}
+
+    def run(eager):
+        eng = Engine(model=path, gpu_memory_utilization=0.5, max_bs=3, enforce_eager=eager, context_len=128, kv_cache_size=300,
+                     dtype=dtype, seed=5)
+        for i, p in prompts.items():
+            eng.add_sequence(i, list(p), SamplingParams(temperature=0.0, ignore_eos=True, max_new_tokens=new[i]))
+        out = {i: [] for i in prompts}
+        while eng.has_unfinished_sequences():
+            for o in eng.step():
+                out[o.seq_id].append(o.new_token_id)
+        stats = dict(eng.model_runner.stats)
+        eng.shutdown()
+        return out, stats
+
+    got, stats = run(False)
+    assert stats["graph_steps"] > 15 and stats["eager_decode_steps"] == 0
+    if dtype == "float32":
+        w = weights_of(cfg, 5)
+        for i, p in prompts.items():
+            assert got[i] == oracle_greedy(w, cfg, p, new[i]), i
+    else:
+        assert got == run(True)[0]
+
+
+def test_generate_entry_point(tmp_path):
+    from nano_vllm_x_amd import LLM, SamplingParams
+    cfg = make_cfg([DEL, PAR], vocab=300)
+    llm = LLM(model_dir(tmp_path, cfg), gpu_memory_utilization=0.5, max_bs=2, enforce_eager=True, context_len=256, kv_cache_size=256,
+              dtype="float32", seed=4)
+    prompt = tokens(11, 300, 1)
+
+    async def run():
+        ids = []
+        async for o in llm.generate(list(prompt), SamplingParams(temperature=0.0, ignore_eos=True, max_new_tokens=5, eos_token_id=0)):
+            ids.append(o.token_id)
+        return ids
+
+    assert asyncio.run(run()) == oracle_greedy(weights_of(cfg, 4), cfg, prompt, 5)
+    llm.shutdown()
+
+
+def test_preempted_sequence_starts_again_from_an_empty_state(tmp_path):
+    from nano_vllm_x_amd.core.common import SamplingParams
+    cfg = make_cfg([MLS, PAR])
+    eng = make_engine(model_dir(tmp_path, cfg), pool=64, max_bs=2, seed=6)
+    w = weights_of(cfg, 6)
+    prompts = {"a": tokens(20, cfg["vocab"], 1), "b": tokens(25, cfg["vocab"], 2)}
+    for i, p in prompts.items():
+        eng.add_sequence(i, list(p), SamplingParams(temperature=0.0, ignore_eos=True, max_new_tokens=14))
+    out = {i: [] for i in prompts}
+    while eng.has_unfinished_sequences():       # 45 + 2 * 14 tokens do not fit 64 slots: the younger sequence is preempted
+        for o in eng.step():
+            out[o.seq_id].append(o.new_token_id)
+    for i, p in prompts.items():
+        assert out[i] == oracle_greedy(w, cfg, p, 14), i
+    eng.shutdown()
+
+
+def test_command_line_generates_what_the_restatement_does(tmp_path):
+    import subprocess
+    import sys
+    cfg = make_cfg([MLS, PAR], vocab=90)
+    path = model_dir(tmp_path, cfg)
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, "-m", "nano_vllm_x_amd", "--model", path, "--prompt-ids", "5,17,3,44", "--prompt-ids", "8",
+                          "--max-new-tokens", "6", "--dtype", "float32", "--kv-cache-size", "128", "--context-len", "64", "--max-bs", "2",
+                          "--seed", "3"], cwd=root, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr[-2000:]
+    lines = [json.loads(x) for x in out.stdout.splitlines() if x.startswith("{")]
+    w = weights_of(cfg, 3)
+    assert [x["prompt"] for x in lines] == [[5, 17, 3, 44], [8]]
+    for x in lines:
+        assert x["generated_ids"] == oracle_greedy(w, cfg, x["prompt"], 6)
+
+
+def test_trace_runner_replays_steps_from_standard_input(tmp_path):
+    """bin/trace_run on a model directory: two requests, portions beside single tokens, one request ended and its id used
+    again; the logits it writes are the restatement's."""
+    import subprocess
+    cfg = make_cfg([PAR, DEL], vocab=80)
+    w = weights_of(cfg, 11)
+    path = model_dir(tmp_path, cfg, w)
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    a, b = tokens(30, 80, 1), tokens(12, 80, 2)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:9], "want": [0, 8]}, {"id": "b", "tokens": b[:1], "want": [0]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": a[9:29], "want": []}, {"id": "b", "tokens": b[1:], "want": [10]}], "end": ["b"]},
+             {"step": 2, "entries": [{"id": "a", "tokens": a[29:], "want": [0]}, {"id": "b", "tokens": a[:5], "want": [4]}], "end": ["a", "b"]}]
+    out_dir = tmp_path / "out"
+    r = subprocess.run([os.path.join(root, "bin", "trace_run"), "--model", path, "--dtype", "float32", "--out", str(out_dir), "--max-tokens", "128"],
+                       input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=600, cwd=root)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [x for x in r.stdout.splitlines() if x.startswith("done")] == ["done 0", "done 1", "done 2"]
+    la, lb = mo.forward(cfg, w, a), mo.forward(cfg, w, b)
+    got = [torch.from_numpy(np.fromfile(out_dir / f"{k}.f32", dtype="<f4").reshape(-1, 80).copy()) for k in range(3)]
+    close(got[0], torch.stack([la[0], la[8], lb[0]]), F32_TOL, "step 0")
+    close(got[1], lb[11:12], F32_TOL, "step 1")
+    close(got[2], torch.stack([la[29], la[4]]), F32_TOL, "step 2")
