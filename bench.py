@@ -42,6 +42,7 @@ METRIC = "output tokens/s (whole node), bench.py 256-req synthetic, Qwen3-0.6B @
 A100_PUBLISHED = 9032.37   # tok/s, 1x A100 40GB, reference README.md:100 (other hardware)
 HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # dense bf16, no sparsity
+FP32_VALU_PEAK_TFLOPS = 157.3    # float32 on the vector units (no matrix cores)
 
 
 def workload(num_seqs: int, max_in: int = 1024, max_out: int = 1024, seed: int = 0):
@@ -497,11 +498,156 @@ def _kernel_table(z, t_pre, n_dec, ctx):
     return rows
 
 
+def _meronex_config(z):
+    """Layers parallel, mlstm, delta in turn; heads of 128 (the recurrences' keys 64 or 128 wide); eight experts of ff / 2 of which a
+    token takes two, so that a token's feed-forward work equals the dense model's."""
+    w, hd = z["width"], z["width"] // 128
+    moe = {"kind": "moe", "expert": {"ff": z["ff"] // 2, "limit": 7.0}, "router": {"experts": 8, "top": 2}}
+    par = {"type": "parallel", "mlp": moe, "mixer": {
+        "left": {"heads": z["heads"], "kv_heads": 8, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "softcap": 30.0,
+                 "rot": {"dims": 64, "base": 1e6, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}},
+        "right": {"heads": w // 64, "dim": 64, "decay_rank": 64}}}
+    mls = {"type": "mlstm", "mlp": moe, "mixer": {"heads": hd, "dim": 64, "vdim": 128, "gate_cap": 15.0}}
+    dlt = {"type": "delta", "mlp": moe, "mixer": {"heads": hd, "kv_heads": max(hd // 2, 1), "dim": 128, "vdim": 128, "conv": 4}}
+    return {"architecture": "Meronex", "vocab": z["vocab"], "width": w, "norm": {"eps": 1e-5, "groups": 4}, "residual_mult": 0.5,
+            "layers": [(par, mls, dlt)[i % 3] for i in range(z["layers"])]}
+
+
+def _meronex_kernel_table(z, t_pre, n_dec, ctx):
+    """Each kernel of Meronex beside the like kernel of Qwen3 (or of the other seq-state model) at the same shape: time, and the
+    fraction of its roofline (HBM bytes it must move at 8 TB/s; attention in prefill: its multiply-adds at the dense bf16 MFMA
+    peak; the recurrences in prefill: their multiply-adds at the float32 vector peak, since their state is float32)."""
+    from nano_vllm_x_amd import ops
+    dev, bf = torch.device("cuda"), torch.bfloat16
+    w, ff, h = z["width"], z["ff"] // 2, z["heads"]
+    hd = w // 128
+    rows = []
+
+    def layout(n_seq, q_len, pos0):
+        p = torch.full((n_seq,), pos0, dtype=torch.int64, device=dev)
+        sl = torch.arange(n_seq, dtype=torch.int32, device=dev)
+        if q_len == 1:
+            return ops.StepLayout(n_seq, n_seq, p, sl)
+        qo = torch.arange(0, n_seq + 1, dtype=torch.int32, device=dev) * q_len
+        return ops.StepLayout(n_seq * q_len, n_seq, p, sl, qo, torch.arange(n_seq, dtype=torch.int32, device=dev).repeat_interleave(q_len))
+
+    def add(name, phase, us, bytes_=None, flops=None, like=None, peak=None):
+        if bytes_:
+            frac, bound = bytes_ / (us * 1e-6) / (HBM_PEAK_GBS * 1e9), "HBM"
+        else:
+            frac, bound = flops / (us * 1e-6) / ((peak or MFMA_BF16_PEAK_TFLOPS) * 1e12), "MFMA" if peak is None else "fp32 VALU"
+        rows.append({"kernel": name, "phase": phase, "us": round(us, 1), "of_roofline": round(frac, 3), "bound": bound, "like": like})
+
+    for phase, (n_seq, q_len, pos0) in (("prefill", (t_pre // 1024, 1024, 0)), ("decode", (n_dec, 1, ctx))):
+        t = n_seq * q_len
+        lay = layout(n_seq, q_len, pos0)
+        reps = 3 if phase == "prefill" else 20
+        y, gate, x = torch.randn(t, w, device=dev).to(bf), torch.randn(t, w, device=dev).to(bf), torch.randn(t, w, device=dev)
+        wv = torch.ones(w, device=dev)
+        # sublayer boundary: reads y and the gate (2 B each) and the stream (4 B), writes the stream (4 B) and the normed rows (2 B)
+        add("gated_residual_norm", phase, _time_us(lambda: ops.gated_residual_norm(x, y=y, gate=gate, gate_bias=wv, mult=0.5, w_norm=wv, groups=4, eps=1e-5)),
+            bytes_=t * w * 14, like="rmsnorm+residual")
+        xb = x.to(bf)
+        add("qwen3 rmsnorm+residual", phase, _time_us(lambda: ops.rmsnorm(y, wv.to(bf), 1e-5, xb)), bytes_=t * w * 8)
+        o32 = torch.randn(t, hd, 128, device=dev)
+        add("head_norm_gate", phase, _time_us(lambda: ops.head_norm_gate(o32, wv, 1e-5, gate=gate, kind="silu")), bytes_=t * w * 8, like="silu_mul")
+        gu = torch.randn(t, 2 * ff, device=dev).to(bf)
+        add("moe_glu", phase, _time_us(lambda: ops.moe_glu(gu, 7.0, 1.702)), bytes_=t * ff * 6, like="silu_mul")
+        add("qwen3 silu_mul", phase, _time_us(lambda: ops.silu_mul(gu)), bytes_=t * ff * 6)
+        # delta: convolution over q | k | v (kv heads hd / 2), then the recurrence
+        gd = max(hd // 2, 1) * 128
+        ch = 2 * gd + hd * 128
+        xq = torch.randn(t, ch + w, device=dev).to(bf)
+        st = torch.zeros(n_seq + 1, 3, ch, device=dev)
+        taps = torch.randn(4, ch, device=dev)
+        add("short_conv_silu", phase, _time_us(lambda: ops.short_conv_silu(xq[:, :ch], taps, st, lay)), bytes_=t * ch * 4 + n_seq * 3 * ch * 8, like="canon_conv")
+        mem = torch.zeros(n_seq + 1, hd, 128, 128, device=dev)
+        ab = torch.randn(t, 2 * hd, device=dev)
+        hz = torch.zeros(hd, device=dev)
+        state_bytes = n_seq * hd * 128 * 128 * 8
+        us = _time_us(lambda: ops.delta_scan(xq, (0, gd, 2 * gd), ab, hz, hz, mem, lay, hd, max(hd // 2, 1), 128, 128), reps)
+        if phase == "prefill":
+            add("delta_scan", phase, us, flops=8.0 * t * hd * 128 * 128, peak=FP32_VALU_PEAK_TFLOPS, like="mingru_scan")
+        else:
+            add("delta_scan", phase, us, bytes_=state_bytes + t * ch * 2, like="mingru_scan")
+        # mlstm: keys 64 wide
+        xm = torch.randn(t, 2 * hd * 64 + 2 * w, device=dev).to(bf)
+        mem2, nrm, pk = torch.zeros(n_seq + 1, hd, 64, 128, device=dev), torch.zeros(n_seq + 1, hd, 64, device=dev), torch.zeros(n_seq + 1, hd, device=dev)
+        gb = torch.zeros(2 * hd, device=dev)
+        us = _time_us(lambda: ops.mlstm_scan(xm, (0, hd * 64, 2 * hd * 64), ab, gb, 15.0, mem2, nrm, pk, lay, hd, 64, 128), reps)
+        if phase == "prefill":
+            add("mlstm_scan", phase, us, flops=6.0 * t * hd * 64 * 128, peak=FP32_VALU_PEAK_TFLOPS, like="mingru_scan")
+        else:
+            add("mlstm_scan", phase, us, bytes_=state_bytes // 2 + t * (2 * hd * 64 + w) * 2, like="mingru_scan")
+        # time mixing: heads of 64
+        h64 = w // 64
+        hm = torch.randn(t, w, device=dev).to(bf)
+        mu = torch.rand(5, w, device=dev)
+        prev = torch.zeros(n_seq + 1, w, device=dev)
+        add("token_shift_mix", phase, _time_us(lambda: ops.token_shift_mix(hm, mu, prev, lay)), bytes_=t * w * 12, like="canon_conv")
+        rkv = torch.randn(3, t, w, device=dev).to(bf)
+        wlog = torch.randn(t, w, device=dev) - 3.0
+        mem3 = torch.zeros(n_seq + 1, h64, 64, 64, device=dev)
+        w0, bonus = torch.zeros(w, device=dev), torch.zeros(h64, 64, device=dev)
+        us = _time_us(lambda: ops.rwkv_scan(rkv[0], rkv[1], rkv[2], wlog, w0, bonus, mem3, lay, h64, 64), reps)
+        if phase == "prefill":
+            add("rwkv_scan", phase, us, flops=6.0 * t * h64 * 64 * 64, peak=FP32_VALU_PEAK_TFLOPS, like="mingru_scan")
+        else:
+            add("rwkv_scan", phase, us, bytes_=n_seq * h64 * 64 * 64 * 8 + t * w * 10, like="mingru_scan")
+        zxg = torch.randn(t, 3 * w, device=dev).to(bf)
+        gs = torch.zeros(n_seq + 1, w, device=dev)
+        add("kabidra mingru_scan", phase, _time_us(lambda: ops.mingru_scan(zxg, gs, lay)), bytes_=t * w * 8 + n_seq * w * 8)
+        # attention: 8 key/value heads of 128, beside paged attention over the same tokens
+        kv_len = pos0 + q_len
+        n_rows = n_seq * kv_len
+        kc, vc = torch.randn(n_rows, 8 * 128, device=dev).to(bf), torch.randn(n_rows, 8 * 128, device=dev).to(bf)
+        idx = torch.arange(n_rows, dtype=torch.int32, device=dev)
+        kv_start = torch.arange(n_seq, dtype=torch.int64, device=dev) * kv_len
+        kvl = torch.full((n_seq,), kv_len, dtype=torch.int32, device=dev)
+        qkv = torch.randn(t, (h + 16) * 128, device=dev).to(bf)
+        pos = (torch.arange(t, device=dev) % q_len + pos0).to(torch.int64)
+        slots = (torch.arange(t, device=dev) // q_len * kv_len + pos).to(torch.int64)
+        from nano_vllm_x_amd.layers.rotary_embedding import rotary_frequencies
+        fr, mag = rotary_frequencies(64, 1e6, {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0})
+        fr = fr.to(dev)
+        add("rope_vnorm_store", phase, _time_us(lambda: ops.rope_vnorm_store(qkv, pos, fr, mag, 64, 1e-5, slots, kc, vc, h, 8, 128, 128)),
+            bytes_=t * (h + 16) * 128 * 2 + t * (h + 16) * 128 * 2, like="qknorm_rope_store")
+        q128 = torch.randn(t, h * 128, device=dev).to(bf)
+        us = _time_us(lambda: ops.softcap_attn(q128, kc, vc, idx, kv_start, kvl, lay, 0.09, 30.0, h, 8, 128, 128), reps)
+        kc4, vc4 = kc.view(n_rows, 8, 128), vc.view(n_rows, 8, 128)
+        if phase == "prefill":
+            pairs = n_seq * q_len * (q_len + 1) // 2
+            add("softcap_attn", phase, us, flops=4.0 * h * 128 * pairs, like="paged_prefill")
+            plan = ops.prefill_plan_ws(n_seq, dev)
+            kv_indptr = torch.arange(0, n_seq + 1, dtype=torch.int32, device=dev) * kv_len
+            ops.prefill_plan(lay.qo_indptr, plan)
+            us = _time_us(lambda: ops.paged_prefill(q128, kc4, vc4, lay.qo_indptr, kv_indptr, idx, plan, h, 8, 0.1), reps=5)
+            add("qwen3 paged_prefill", phase, us, flops=4.0 * h * 128 * pairs)
+        else:
+            add("softcap_attn", phase, us, bytes_=n_rows * 8 * 128 * 2 * 2 + 2 * t * h * 128 * 2, like="paged_decode")
+            ws = ops.DecodeWorkspace(n_seq, h, 8, dev)
+            ops.decode_plan(kvl, kv_start, ws)
+            us = _time_us(lambda: ops.paged_decode(q128, kc4, vc4, idx, n_seq, ws, 0.1))
+            add("qwen3 paged_decode", phase, us, bytes_=n_rows * 8 * 128 * 2 * 2 + 2 * t * h * 128 * 2)
+        # experts: eight of ff / 2, two a token
+        if phase == "decode":
+            w_gu, w_d = torch.randn(8, 2 * ff, w, device=dev).to(bf) * 0.02, torch.randn(8, w, ff, device=dev).to(bf) * 0.02
+            eidx, wts = ops.moe_route(torch.randn(t, 8, device=dev), 2)
+            us = _time_us(lambda: ops.moe_expert_rows(hm, eidx, wts, w_gu, w_d, 7.0, 1.702))
+            add("moe_expert_rows", phase, us, bytes_=min(t * 2, 8) * 3 * ff * w * 2, like="(library products of the dense feed-forward)")
+    return rows
+
+
+ARCHS = {"kabidra": (lambda z: _kabidra_config(z), lambda *a: _kernel_table(*a), "Kabidra"),
+         "meronex": (lambda z: _meronex_config(z), lambda *a: _meronex_kernel_table(*a), "Meronex")}
+
+
 def arch_compare(args):
     import tempfile
 
     torch.cuda.set_device(0)
-    result = {"metric": "prefill and decode tokens/s, Kabidra beside Qwen3 at equal width, depth, feed-forward and vocabulary",
+    make_config, kernel_table, title = ARCHS[args.arch]
+    result = {"metric": f"prefill and decode tokens/s, {title} beside Qwen3 at equal width, depth, feed-forward and vocabulary",
               "dtype": "bf16", "data": "synthetic (random token ids, random-init weights)", "n_gpus": 1,
               "workload": {"prefill": f"{args.arch_seqs} prompts of {args.arch_prompt} tokens in one step",
                            "decode": f"{args.arch_seqs} sequences, {args.arch_new} steps from context {args.arch_prompt}"},
@@ -510,7 +656,7 @@ def arch_compare(args):
         z = ARCH_SIZES[name]
         entry = {"geometry": z}
         with tempfile.TemporaryDirectory() as tmp:
-            for model, cfg in (("kabidra", _kabidra_config(z)), ("qwen3", _qwen3_config(z))):
+            for model, cfg in ((args.arch, make_config(z)), ("qwen3", _qwen3_config(z))):
                 d = os.path.join(tmp, model)
                 os.makedirs(d)
                 with open(os.path.join(d, "config.json"), "w") as f:
@@ -518,7 +664,7 @@ def arch_compare(args):
                 entry[model] = _serve_once(d, args.arch_seqs, args.arch_prompt, args.arch_new, args.enforce_eager)
                 print(f"[arch-compare] {name} {model}: {entry[model]}", file=sys.stderr, flush=True)
         with torch.inference_mode():
-            entry["kernels"] = _kernel_table(z, args.arch_seqs * args.arch_prompt, args.arch_seqs, args.arch_prompt)
+            entry["kernels"] = kernel_table(z, args.arch_seqs * args.arch_prompt, args.arch_seqs, args.arch_prompt)
         result["sizes"][name] = entry
     print(json.dumps(result), flush=True)
 
@@ -526,8 +672,9 @@ def arch_compare(args):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--arch-compare", action="store_true",
-                    help="instead of the headline workload: prefill and decode rates of Kabidra beside Qwen3 at equal sizes, and "
+                    help="instead of the headline workload: prefill and decode rates of the design named by --arch beside Qwen3 at equal sizes, and "
                          "each of its kernels beside the like Qwen3 kernel against its roofline (one JSON line)")
+    ap.add_argument("--arch", choices=sorted(ARCHS), default="kabidra", help="the design that --arch-compare puts beside Qwen3")
     ap.add_argument("--arch-sizes", default="w1024,w2048,w4096")
     ap.add_argument("--arch-seqs", type=int, default=16)
     ap.add_argument("--arch-prompt", type=int, default=1024)

@@ -44,7 +44,7 @@ typedef void* nvx_stream_t;
  *   8: layers with a 32-bit residual stream and per-sequence state (`nvx_boundary_norm`, `nvx_canon_conv`, `nvx_relu2`,
  *      `nvx_mingru_scan`) and latent attention (`nvx_latent_prep`, `nvx_latent_attn`) added.
  *   9: nvx_boundary_norm can apply the convolution of a decode step in the same launch. */
-#define NVX_ABI_VERSION 10
+#define NVX_ABI_VERSION 11
 
 /* Library identification and diagnostics. */
 int nvx_abi_version(void);
@@ -534,7 +534,10 @@ int nvx_latent_attn(const void* q, const void* cache, int fmt, const int32_t* kv
  *     nvx_moe_expert_rows_max_width(ff)).
  * nvx_moe_scatter_rows:  xs[dst[r]] = wts[r] * h[r / top] for every (token, choice) pair r.
  * nvx_moe_glu:  y[r][j] = the expert's activation of (gu[r][j], gu[r][ff + j]).
- * nvx_moe_gather_rows:  out[t] = sum_k ys[dst[t * top + k]]. */
+ * nvx_moe_gather_rows:  out[t] = sum_k ys[dst[t * top + k]].
+ * nvx_skinny_proj:  out[t][n] = sum_k w[n][k] * f(x[t][k]) in float32, f = identity (in_act 0) or tanh (1); w float32 (n_out,
+ *     k_in), x in the format `fmt`.  Meant for few outputs (gate and router logits) or few inputs (the second half of a low-rank
+ *     map); one fixed summation order, no workspace. */
 int nvx_gated_residual_norm(const void* y, int64_t y_stride, const void* y2, int64_t y2_stride, const float* w_y,
                             const float* w_y2, const void* gate, int64_t gate_stride, const float* gate_bias, int fmt,
                             float mult, float* x, const float* w_norm, int groups, float eps, void* h_out, int64_t n_tok,
@@ -577,6 +580,8 @@ int nvx_moe_scatter_rows(const void* h, int64_t h_stride, int fmt, const float* 
 int nvx_moe_glu(const void* gu, int fmt, float limit, float alpha, void* y, int64_t rows, int64_t ff, nvx_stream_t stream);
 int nvx_moe_gather_rows(const void* ys, int fmt, const int64_t* dst, int64_t top, void* out, int64_t n_tok, int64_t width,
                         nvx_stream_t stream);
+int nvx_skinny_proj(const void* x, int64_t x_stride, int fmt, const float* w, int in_act, float* out, int64_t n_tok,
+                    int64_t n_out, int64_t k_in, nvx_stream_t stream);
 
 #ifdef __cplusplus
 }

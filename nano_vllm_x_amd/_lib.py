@@ -116,6 +116,7 @@ SIGNATURES = {
     "nvx_moe_scatter_rows": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_vp, _c_vp, _c_i64, _c_vp, _c_i64, _c_i64, _c_vp]),
     "nvx_moe_glu": (_c_i32, [_c_vp, _c_i32, _c_f32, _c_f32, _c_vp, _c_i64, _c_i64, _c_vp]),
     "nvx_moe_gather_rows": (_c_i32, [_c_vp, _c_i32, _c_vp, _c_i64, _c_vp, _c_i64, _c_i64, _c_vp]),
+    "nvx_skinny_proj": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_vp, _c_i32, _c_vp, _c_i64, _c_i64, _c_i64, _c_vp]),
 }
 
 _lib = None

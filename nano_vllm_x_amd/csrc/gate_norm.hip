@@ -82,9 +82,83 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __rest
     }
 }
 
+
+// Projections onto FEW outputs or from FEW inputs, in float32: gate and router logits (outputs = heads or experts), the two
+// halves of a low-rank decay.  out[t][n] = sum_k W[n][k] * f(x[t][k]), f = identity or tanh; W float32 (n_out, k_in).  A
+// workgroup takes TOK tokens: their inputs wait in LDS as float32, every weight is read once for the TOK of them.  Wide
+// inputs: a wave per output, lanes over k.  Narrow inputs (k_in < 256): a thread per output.  No workspace, no atomics: the
+// sums have one order, and the launch can be captured.
+template <typename A, int TOK>
+__global__ __launch_bounds__(256) void skinny_proj_kernel(const A* __restrict__ x, int64_t x_stride, const float* __restrict__ w,
+                                                         int in_act, float* __restrict__ out, int64_t n_tok, int n_out, int k_in) {
+    extern __shared__ float xs[];      // TOK rows of k_in
+    const int64_t t0 = (int64_t)blockIdx.x * TOK;
+    const int nt = (int)(n_tok - t0 < TOK ? n_tok - t0 : TOK);
+    for (int i = threadIdx.x; i < TOK * k_in; i += 256) {
+        const int tt = i / k_in, k = i % k_in;
+        float v = tt < nt ? ld_f(x, (t0 + tt) * x_stride + k) : 0.f;
+        xs[i] = in_act == 1 ? tanhf(v) : v;
+    }
+    __syncthreads();
+    if (k_in >= 256) {
+        const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+        for (int n = wave; n < n_out; n += 4) {
+            const float* wr = w + (int64_t)n * k_in;
+            float acc[TOK];
+#pragma unroll
+            for (int tt = 0; tt < TOK; ++tt) acc[tt] = 0.f;
+            for (int k = lane; k < k_in; k += 64) {
+                const float wv = wr[k];
+#pragma unroll
+                for (int tt = 0; tt < TOK; ++tt) acc[tt] += wv * xs[tt * k_in + k];
+            }
+#pragma unroll
+            for (int tt = 0; tt < TOK; ++tt) {
+                const float sum = wave_sum(acc[tt]);
+                if (lane == 0 && tt < nt) out[(t0 + tt) * n_out + n] = sum;
+            }
+        }
+    } else {
+        for (int n = threadIdx.x; n < n_out; n += 256) {
+            const float* wr = w + (int64_t)n * k_in;
+            float acc[TOK];
+#pragma unroll
+            for (int tt = 0; tt < TOK; ++tt) acc[tt] = 0.f;
+            for (int k = 0; k < k_in; ++k) {
+                const float wv = wr[k];
+#pragma unroll
+                for (int tt = 0; tt < TOK; ++tt) acc[tt] += wv * xs[tt * k_in + k];
+            }
+#pragma unroll
+            for (int tt = 0; tt < TOK; ++tt)
+                if (tt < nt) out[(t0 + tt) * n_out + n] = acc[tt];
+        }
+    }
+}
+
 }  // namespace NVX_NS
 
 using namespace NVX_NS;
+
+extern "C" int nvx_skinny_proj(const void* x, int64_t x_stride, int fmt, const float* w, int in_act, float* out, int64_t n_tok,
+                               int64_t n_out, int64_t k_in, nvx_stream_t stream) {
+    NVX_REQUIRE(fmt >= 0 && fmt <= 2 && (in_act == 0 || in_act == 1), NVX_EINVAL, "nvx_skinny_proj: fmt must be 0..2, in_act 0 or 1");
+    NVX_REQUIRE(n_tok >= 0 && n_out > 0 && n_out < (1 << 24) && k_in > 0 && k_in <= 12288 && x_stride >= k_in, NVX_EINVAL,
+                "nvx_skinny_proj: bad sizes (at most 12288 inputs)");
+    if (n_tok == 0) return NVX_OK;
+    NVX_REQUIRE(x && w && out, NVX_EINVAL, "nvx_skinny_proj: null pointer");
+    if (k_in <= 3072) {
+        const int64_t blocks = (n_tok + 3) / 4;
+        NVX_REQUIRE(blocks < (1ll << 31), NVX_EINVAL, "nvx_skinny_proj: too many tokens");
+        NVX_FMT_CALL(fmt, hipLaunchKernelGGL((skinny_proj_kernel<A_, 4>), dim3((unsigned)blocks), dim3(256), (size_t)(4 * k_in) * sizeof(float),
+                                             (hipStream_t)stream, (const A_*)x, x_stride, w, in_act, out, n_tok, (int)n_out, (int)k_in));
+    } else {
+        NVX_REQUIRE(n_tok < (1ll << 31), NVX_EINVAL, "nvx_skinny_proj: too many tokens");
+        NVX_FMT_CALL(fmt, hipLaunchKernelGGL((skinny_proj_kernel<A_, 1>), dim3((unsigned)n_tok), dim3(256), (size_t)k_in * sizeof(float),
+                                             (hipStream_t)stream, (const A_*)x, x_stride, w, in_act, out, n_tok, (int)n_out, (int)k_in));
+    }
+    return nvx_check_launch("nvx_skinny_proj");
+}
 
 extern "C" int nvx_gated_residual_norm(const void* y, int64_t y_stride, const void* y2, int64_t y2_stride, const float* w_y,
                                        const float* w_y2, const void* gate, int64_t gate_stride, const float* gate_bias, int fmt,

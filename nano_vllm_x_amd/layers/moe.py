@@ -30,7 +30,7 @@ class SigmoidInputMoE(nn.Module):
 
     def forward(self, h: torch.Tensor, decode_step: bool = False) -> torch.Tensor:
         t = h.shape[0]
-        idx, wts = ops.moe_route(F.linear(h.float(), self.router), self.top)
+        idx, wts = ops.moe_route(ops.skinny_proj(h, self.router), self.top)
         if self._rows_fit is None:
             self._rows_fit = ops.moe_expert_rows_fits(self.width, self.ff)
         if self._rows_fit and (decode_step or t <= self.ROWS_PATH_TOKENS):

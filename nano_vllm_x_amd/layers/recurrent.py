@@ -56,7 +56,7 @@ class MLSTM(nn.Module):
     def forward(self, h: torch.Tensor, md) -> torch.Tensor:
         hd, he, n = self.heads * self.dim, self.heads * self.vdim, self.state_name
         x = self.qkvg_proj(h)
-        gates = F.linear(h.float(), self.gate_w)
+        gates = ops.skinny_proj(h, self.gate_w)
         o = ops.mlstm_scan(x, (0, hd, 2 * hd), gates, self.gate_b, self.gate_cap, md.cache.state((n, "S")), md.cache.state((n, "n")),
                            md.cache.state((n, "m")), md.layout, self.heads, self.dim, self.vdim)
         y = ops.head_norm_gate(o, self.norm, self.eps, gate=x[:, 2 * hd + he:], kind="sigmoid")
@@ -93,7 +93,7 @@ class GatedDelta(nn.Module):
         gd, n = self.kv_heads * self.dim, self.state_name
         x = self.qkvg_proj(h)
         xc = ops.short_conv_silu(x[:, :self.conv_ch], self.conv_w, md.cache.state((n, "conv")) if self.taps > 1 else None, md.layout)
-        ab = F.linear(h.float(), self.ab_w)
+        ab = ops.skinny_proj(h, self.ab_w)
         o = ops.delta_scan(xc, (0, gd, 2 * gd), ab, self.a_log, self.dt_bias, md.cache.state((n, "S")), md.layout, self.heads, self.kv_heads,
                            self.dim, self.vdim)
         y = ops.head_norm_gate(o, self.norm, self.eps, gate=x[:, self.conv_ch:], kind="silu")
@@ -106,7 +106,7 @@ class TimeMix(nn.Module):
     w = exp(-exp(W_w2 tanh(W_w1 blend_w) + w0)) per head and key channel.  Per head o = (S + diag(bonus) k v^T)^T r, then
     S <- diag(w) S + k v^T.  Each head's o is divided by its root mean square, times `norm`, times the gate, then W_o.
     State: S (float32) and the predecessor's input row.  The four wide projections are one batched matrix product; the
-    decay's two small ones are float32."""
+    decay's two small ones are float32 (ops.skinny_proj, the tanh applied as the second one reads its input)."""
 
     MIXES = ("r", "k", "v", "g", "w")
 
@@ -128,7 +128,7 @@ class TimeMix(nn.Module):
         n = self.state_name
         blends = ops.token_shift_mix(h, self.mu, md.cache.state((n, "prev")), md.layout)          # (5, T, width)
         proj = torch.bmm(blends[:4], self.rkvg.transpose(1, 2))                                    # (4, T, heads * dim)
-        wlog = F.linear(torch.tanh(F.linear(blends[4].float(), self.w1)), self.w2)
+        wlog = ops.skinny_proj(ops.skinny_proj(blends[4], self.w1), self.w2, in_act="tanh")
         o = ops.rwkv_scan(proj[0], proj[1], proj[2], wlog, self.w0, self.bonus, md.cache.state((n, "S")), md.layout, self.heads, self.dim)
         y = ops.head_norm_gate(o, self.norm, self.eps, gate=proj[3], kind="silu")
         return self.o_proj(y)

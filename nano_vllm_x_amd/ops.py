@@ -1139,3 +1139,17 @@ def moe_gather_rows(ys, dst):
     lib = _lib.load()
     _lib.check(lib.nvx_moe_gather_rows(_ptr(ys), _fmt(ys), _ptr(dst), top, _ptr(out), t, ys.shape[1], _stream()), "nvx_moe_gather_rows")
     return out
+
+
+def skinny_proj(x, w, in_act: str = "none"):
+    """out = f(x) @ w.T in float32, f = identity or tanh: x (T, k_in) in any activation format (rows may be a slice of wider
+    rows), w (n_out, k_in) float32.  For few outputs (gate and router logits) or few inputs; one fixed summation order and
+    no workspace, so a captured launch replays to the same bits."""
+    _dev(x, w)
+    _f32c(w, "skinny_proj: w")
+    _need(x.dim() == 2 and x.stride(1) == 1 and w.dim() == 2 and w.shape[1] == x.shape[1], "skinny_proj: x must be (T, k_in), w (n_out, k_in)")
+    out = torch.empty((x.shape[0], w.shape[0]), dtype=F32, device=x.device)
+    lib = _lib.load()
+    _lib.check(lib.nvx_skinny_proj(_ptr(x), x.stride(0), _fmt(x), _ptr(w), {"none": 0, "tanh": 1}[in_act], _ptr(out), x.shape[0], w.shape[0],
+                                   x.shape[1], _stream()), "nvx_skinny_proj")
+    return out

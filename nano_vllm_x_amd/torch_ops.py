@@ -89,6 +89,7 @@ _DEFS = {
     "moe_scatter_rows": "(Tensor h, Tensor wts, Tensor dst) -> Tensor",
     "moe_glu": "(Tensor gu, float limit, float alpha) -> Tensor",
     "moe_gather_rows": "(Tensor ys, Tensor dst) -> Tensor",
+    "skinny_proj": "(Tensor x, Tensor w, str in_act) -> Tensor",
 }
 for _name, _sig in _DEFS.items():
     _LIB.define(_name + _sig)
@@ -305,6 +306,10 @@ def _moe_glu(gu, limit, alpha):
 
 def _moe_gather_rows(ys, dst):
     return ops.moe_gather_rows(ys, dst)
+
+
+def _skinny_proj(x, w, in_act):
+    return ops.skinny_proj(x, w, in_act)
 
 
 for _name in _DEFS:

@@ -157,6 +157,19 @@ def test_head_norm_and_output_gate(kind, shared):
     assert torch.allclose(got.cpu(), want, atol=1e-5)
 
 
+@pytest.mark.parametrize("fmt", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("k_in,n_out", [(70, 300), (1024, 6), (3100, 5), (256, 64), (5, 1)])
+def test_small_float32_projections(fmt, k_in, n_out):
+    from nano_vllm_x_amd import ops
+    g = torch.Generator().manual_seed(k_in)
+    wide = torch.randn(7, k_in + 9, generator=g).to(fmt)
+    x, w = wide[:, 4:4 + k_in], torch.randn(n_out, k_in, generator=g)
+    got = ops.skinny_proj(wide.cuda()[:, 4:4 + k_in], w.cuda())
+    assert got.dtype == torch.float32
+    close(got.cpu(), x.double() @ w.double().T, 2e-6, "plain")
+    close(ops.skinny_proj(wide.cuda()[:, 4:4 + k_in], w.cuda(), in_act="tanh").cpu(), torch.tanh(x.double()) @ w.double().T, 2e-6, "tanh")
+
+
 @pytest.mark.parametrize("taps", [1, 2, 3, 6])
 def test_short_convolution_continues_over_cuts_and_reused_slots(taps):
     """Two sequences in slots that are not in order, cut into steps of 1, 2, taps - 1, taps and more tokens; a third
