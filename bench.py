@@ -661,8 +661,10 @@ def arch_compare(args):
                 os.makedirs(d)
                 with open(os.path.join(d, "config.json"), "w") as f:
                     json.dump(cfg, f)
+                print(f"[arch-compare] {name} {model}: serving", file=sys.stderr, flush=True)
                 entry[model] = _serve_once(d, args.arch_seqs, args.arch_prompt, args.arch_new, args.enforce_eager)
                 print(f"[arch-compare] {name} {model}: {entry[model]}", file=sys.stderr, flush=True)
+        print(f"[arch-compare] {name}: kernels one by one", file=sys.stderr, flush=True)
         with torch.inference_mode():
             entry["kernels"] = kernel_table(z, args.arch_seqs * args.arch_prompt, args.arch_seqs, args.arch_prompt)
         result["sizes"][name] = entry
