@@ -44,7 +44,7 @@ typedef void* nvx_stream_t;
  *   8: layers with a 32-bit residual stream and per-sequence state (`nvx_boundary_norm`, `nvx_canon_conv`, `nvx_relu2`,
  *      `nvx_mingru_scan`) and latent attention (`nvx_latent_prep`, `nvx_latent_attn`) added.
  *   9: nvx_boundary_norm can apply the convolution of a decode step in the same launch. */
-#define NVX_ABI_VERSION 11
+#define NVX_ABI_VERSION 12
 
 /* Library identification and diagnostics. */
 int nvx_abi_version(void);
@@ -511,7 +511,9 @@ int nvx_latent_attn(const void* q, const void* cache, int fmt, const int32_t* kv
  *     (float32, heads each; gate_bias likewise).  i' = cap tanh((i + b_i) / cap), f' = logsigmoid(cap tanh((f + b_f) / cap));
  *     m <- max(f' + m_old, i');  S <- e^(f' + m_old - m) S + e^(i' - m) k v^T;  n likewise with k;
  *     out[t] = S^T q dim^(-1/2) / (max(|n . q dim^(-1/2)|, e^(-m)) + 1e-6)   (float32, heads * vdim).  S (slots, heads, dim, vdim),
- *     N (slots, heads, dim), M (slots, heads) are continued and written back; all start from zero.  dim <= 512.
+ *     N (slots, heads, dim), M (slots, heads) are continued and written back; all start from zero.  dim <= 512.  They are read
+ *     through N_in / M_in: the same pointers where a head is one column block (nvx_scan_column_blocks(dim, vdim) == 1), copies
+ *     taken before the launch otherwise (a column block that starts late must not read what the first one has written).
  * nvx_delta_scan:  x[t] holds q at q_off, k at k_off (kv_heads * dim) and v at v_off (heads * vdim); ab[t] = [a | b] (float32, heads
  *     each).  q, k <- unit length per head (x / sqrt(sum x^2 + 1e-6)), q also times dim^(-1/2);  g = exp(-exp(a_log) softplus(a +
  *     dt_bias)), beta = sigmoid(b);  S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  out[t] = S^T q.  Head h reads q/k head
@@ -550,8 +552,10 @@ int nvx_short_conv_silu(const void* x, int64_t x_stride, int fmt, const float* w
 int nvx_token_shift_mix(const void* h, int64_t h_stride, int fmt, const float* mu, int n_mix, float* state, int64_t n_slots,
                         const int32_t* tok_seq, const int32_t* qo_indptr, const int64_t* pos0, const int32_t* state_slot,
                         void* out, int64_t n_tok, int64_t n_seq, int64_t width, nvx_stream_t stream);
+int64_t nvx_scan_column_blocks(int64_t dim, int64_t vdim);
 int nvx_mlstm_scan(const void* x, int64_t x_stride, int fmt, int64_t q_off, int64_t k_off, int64_t v_off, const float* gates,
-                   const float* gate_bias, float cap, float* S, float* N, float* M, int64_t n_slots, const int32_t* qo_indptr,
+                   const float* gate_bias, float cap, float* S, const float* N_in, const float* M_in, float* N, float* M,
+                   int64_t n_slots, const int32_t* qo_indptr,
                    const int64_t* pos0, const int32_t* state_slot, float* out, int64_t n_tok, int64_t n_seq, int64_t heads,
                    int64_t dim, int64_t vdim, nvx_stream_t stream);
 int nvx_delta_scan(const void* x, int64_t x_stride, int fmt, int64_t q_off, int64_t k_off, int64_t v_off, const float* ab,

@@ -99,7 +99,8 @@ SIGNATURES = {
                                      _c_i64, _c_vp]),
     "nvx_token_shift_mix": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_vp, _c_i32, _c_vp, _c_i64, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_i64,
                                      _c_i64, _c_vp]),
-    "nvx_mlstm_scan": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_i64, _c_i64, _c_i64, _c_vp, _c_vp, _c_f32, _c_vp, _c_vp, _c_vp, _c_i64, _c_vp, _c_vp,
+    "nvx_scan_column_blocks": (_c_i64, [_c_i64, _c_i64]),
+    "nvx_mlstm_scan": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_i64, _c_i64, _c_i64, _c_vp, _c_vp, _c_f32, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_vp, _c_vp,
                                 _c_vp, _c_vp, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_vp]),
     "nvx_delta_scan": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_i64, _c_i64, _c_i64, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_vp, _c_vp, _c_vp, _c_vp,
                                 _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_vp]),

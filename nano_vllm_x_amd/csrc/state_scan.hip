@@ -141,10 +141,13 @@ __device__ __forceinline__ void unit_rows(float* dst, int nt, int dim, int p_lan
 // (heads each, float32), gate_bias likewise.  i = cap tanh(. / cap), f = logsigmoid(cap tanh(. / cap));
 //   m' = max(f + m, i);  S <- e^(f + m - m') S + e^(i - m') k v^T;  n likewise with k;  o = S^T q / (max(|n.q|, e^(-m')) + 1e-6)
 // with q scaled by dim^(-1/2); m starts at 0.  S: (slots, heads, dim, vdim), n: (slots, heads, dim), m: (slots, heads).
+// Every column block of a head reads n and m (N_in, M_in) and the first one writes them (N, M): where a head has more than one
+// column block the caller hands in copies to read from, since a block that starts late must not see the new values.
 template <typename A>
 __global__ __launch_bounds__(256) void mlstm_scan_kernel(const A* __restrict__ x, int64_t x_stride, int q_off, int k_off, int v_off,
                                                         const float* __restrict__ gates, const float* __restrict__ gate_bias, float cap,
-                                                        float* __restrict__ S, float* __restrict__ N, float* __restrict__ M,
+                                                        float* __restrict__ S, const float* __restrict__ N_in, const float* __restrict__ M_in,
+                                                        float* __restrict__ N, float* __restrict__ M,
                                                         const int32_t* __restrict__ qo_indptr, const int64_t* __restrict__ pos0,
                                                         const int32_t* __restrict__ state_slot, float* __restrict__ out, int heads, int dim,
                                                         int vdim, int p_lanes) {
@@ -161,6 +164,7 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(const A* __restrict__ x
     const ScanThread th = scan_thread(p_lanes, vdim);
     float* Sp = S + ((int64_t)sp.slot * heads + hd) * dim * vdim;
     float* Np = N + ((int64_t)sp.slot * heads + hd) * dim;
+    const float* Np_in = N_in + ((int64_t)sp.slot * heads + hd) * dim;
     float s[KR], nn[KR];
     float m = 0.f;
     const bool cont = sp.pos0 > 0;
@@ -169,9 +173,9 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(const A* __restrict__ x
         const int row = th.r0 + r;
         const bool in = cont && row < dim;
         s[r] = (in && th.active) ? Sp[(int64_t)row * vdim + th.e] : 0.f;
-        nn[r] = in ? Np[row] : 0.f;
+        nn[r] = in ? Np_in[row] : 0.f;
     }
-    if (cont) m = M[(int64_t)sp.slot * heads + hd];
+    if (cont) m = M_in[(int64_t)sp.slot * heads + hd];
     zero_rows(sq, 2 * TB * rs);
     const float q_mul = 1.0f / sqrtf((float)dim);
     for (int64_t t0 = 0; t0 < sp.n; t0 += TB) {
@@ -422,8 +426,15 @@ extern "C" int nvx_token_shift_mix(const void* h, int64_t h_stride, int fmt, con
     return nvx_check_launch("nvx_token_shift_mix");
 }
 
+extern "C" int64_t nvx_scan_column_blocks(int64_t dim, int64_t vdim) {
+    ScanLaunch g;
+    if (dim <= 0 || vdim <= 0 || !scan_launch(dim, vdim, &g)) return 0;
+    return (vdim + g.cb - 1) / g.cb;
+}
+
 extern "C" int nvx_mlstm_scan(const void* x, int64_t x_stride, int fmt, int64_t q_off, int64_t k_off, int64_t v_off, const float* gates,
-                              const float* gate_bias, float cap, float* S, float* N, float* M, int64_t n_slots, const int32_t* qo_indptr,
+                              const float* gate_bias, float cap, float* S, const float* N_in, const float* M_in, float* N, float* M,
+                              int64_t n_slots, const int32_t* qo_indptr,
                               const int64_t* pos0, const int32_t* state_slot, float* out, int64_t n_tok, int64_t n_seq, int64_t heads,
                               int64_t dim, int64_t vdim, nvx_stream_t stream) {
     NVX_LAYOUT_OK("nvx_mlstm_scan");
@@ -431,13 +442,15 @@ extern "C" int nvx_mlstm_scan(const void* x, int64_t x_stride, int fmt, int64_t 
     NVX_REQUIRE(heads > 0 && heads <= 65535 && dim > 0 && vdim > 0 && vdim < (1 << 24) && n_slots >= 0 && cap > 0.f, NVX_EINVAL,
                 "nvx_mlstm_scan: bad sizes");
     NVX_REQUIRE(scan_launch(dim, vdim, &g), NVX_EUNSUPPORTED, "nvx_mlstm_scan: key size above 512");
-    NVX_REQUIRE(x && gates && gate_bias && S && N && M && out, NVX_EINVAL, "nvx_mlstm_scan: null pointer");
+    NVX_REQUIRE(x && gates && gate_bias && S && N && M && N_in && M_in && out, NVX_EINVAL, "nvx_mlstm_scan: null pointer");
     NVX_REQUIRE(q_off >= 0 && k_off >= 0 && v_off >= 0 && x_stride >= q_off + heads * dim && x_stride >= k_off + heads * dim &&
                     x_stride >= v_off + heads * vdim, NVX_EINVAL, "nvx_mlstm_scan: q, k or v lies outside a row");
     const size_t lds = (size_t)(2 * TB * g.p_lanes * KS + TB * g.cb + 2 * TB) * sizeof(float);
     const dim3 grid((unsigned)((vdim + g.cb - 1) / g.cb), (unsigned)heads, (unsigned)n_seq);
+    NVX_REQUIRE(grid.x == 1 || (N_in != N && M_in != M), NVX_EINVAL,
+                "nvx_mlstm_scan: a head with several column blocks reads its normaliser and maximum from copies");
     NVX_FMT_CALL(fmt, hipLaunchKernelGGL(mlstm_scan_kernel<A_>, grid, dim3(g.threads), lds, (hipStream_t)stream, (const A_*)x, x_stride, (int)q_off,
-                                         (int)k_off, (int)v_off, gates, gate_bias, cap, S, N, M, qo_indptr, pos0, state_slot, out, (int)heads,
+                                         (int)k_off, (int)v_off, gates, gate_bias, cap, S, N_in, M_in, N, M, qo_indptr, pos0, state_slot, out, (int)heads,
                                          (int)dim, (int)vdim, g.p_lanes));
     return nvx_check_launch("nvx_mlstm_scan");
 }

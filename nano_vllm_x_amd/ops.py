@@ -978,8 +978,12 @@ def mlstm_scan(x, offsets, gates, gate_bias, cap: float, mem, norm, peak, layout
     _need(mem.shape == (n_slots, heads, dim, vdim) and norm.shape == (n_slots, heads, dim) and peak.shape == (n_slots, heads), "mlstm_scan: state shapes")
     out = torch.empty((t, heads, vdim), dtype=F32, device=x.device)
     lib = _lib.load()
+    # a head whose value columns take several workgroups: all of them read the normaliser and the maximum, the first writes them
+    # back, so they read from copies (a workgroup that starts late must not see the new values)
+    several = lib.nvx_scan_column_blocks(dim, vdim) != 1
+    norm_in, peak_in = (norm.clone(), peak.clone()) if several else (norm, peak)
     _lib.check(lib.nvx_mlstm_scan(_ptr(x), x.stride(0), _fmt(x), offsets[0], offsets[1], offsets[2], _ptr(gates), _ptr(gate_bias), float(cap),
-                                  _ptr(mem), _ptr(norm), _ptr(peak), n_slots, *_layout_args(layout), _ptr(out), t, layout.n_seq, heads, dim, vdim,
+                                  _ptr(mem), _ptr(norm_in), _ptr(peak_in), _ptr(norm), _ptr(peak), n_slots, *_layout_args(layout), _ptr(out), t, layout.n_seq, heads, dim, vdim,
                                   _stream()), "nvx_mlstm_scan")
     return out
 
