@@ -2,8 +2,9 @@
 //   - nvx_moe_route: the `top` largest router logits of every token -> expert ids and sigmoid scores (float32);
 //   - nvx_moe_expert_rows: a token's experts evaluated row by row of their weights (a workgroup per token): the form for
 //     steps of few tokens, where every chosen expert's weights have to be streamed once per token anyway;
-//   - nvx_moe_scatter_rows / nvx_moe_glu / nvx_moe_gather_rows: the pieces around per-expert matrix products for steps of
-//     many tokens (scaled inputs gathered into expert order, the gated activation, the tokens' results summed back).
+//   - nvx_moe_order / nvx_moe_scatter_rows / nvx_moe_glu / nvx_moe_gather_rows: the pieces around per-expert matrix products
+//     for steps of many tokens (the expert order of the (token, choice) pairs and the experts' counts, scaled inputs gathered
+//     into that order, the gated activation, the tokens' results summed back).
 // Expert:  g = min(W_gate x, limit), u = clamp(W_up x, -limit, limit), y = g sigmoid(alpha g) (u + 1), out = W_down y.
 #include "fmt_dev.h"
 
@@ -114,9 +115,55 @@ __global__ __launch_bounds__(256) void moe_gather_rows_kernel(const A* __restric
     }
 }
 
+
+// Expert order of the (token, choice) pairs: dst[r] = position of pair r when the pairs are sorted by expert, pairs of one
+// expert keeping their order; counts[e] = pairs of expert e.  One workgroup: a thread takes a contiguous run of pairs, counts
+// them per expert into LDS (cnt[e][thread]), the prefix sums over (expert, thread) give every thread its first position per
+// expert, and a second walk over the same run hands the positions out.  n_exp * 256 counters must fit LDS.
+__global__ __launch_bounds__(256) void moe_order_kernel(const int32_t* __restrict__ idx, int64_t n, int n_exp, int64_t* __restrict__ dst,
+                                                       int32_t* __restrict__ counts) {
+    extern __shared__ int cnt[];      // n_exp rows of 256, then n_exp bases
+    int* base = cnt + n_exp * 256;
+    const int tid = threadIdx.x;
+    const int64_t per = (n + 255) / 256, lo = tid * per, hi = lo + per < n ? lo + per : n;
+    for (int e = 0; e < n_exp; ++e) cnt[e * 256 + tid] = 0;
+    for (int64_t r = lo; r < hi; ++r) {
+        const int e = idx[r];
+        if (e >= 0 && e < n_exp) cnt[e * 256 + tid] += 1;
+    }
+    __syncthreads();
+    for (int e = tid; e < n_exp; e += 256) {       // a thread per expert: exclusive prefix over the threads' counts
+        int run = 0;
+        for (int j = 0; j < 256; ++j) { const int c = cnt[e * 256 + j]; cnt[e * 256 + j] = run; run += c; }
+        base[e] = run;
+        counts[e] = run;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int run = 0;
+        for (int e = 0; e < n_exp; ++e) { const int c = base[e]; base[e] = run; run += c; }
+    }
+    __syncthreads();
+    for (int64_t r = lo; r < hi; ++r) {
+        const int e = idx[r];
+        if (e >= 0 && e < n_exp) dst[r] = base[e] + cnt[e * 256 + tid]++;
+    }
+}
+
 }  // namespace NVX_NS
 
 using namespace NVX_NS;
+
+extern "C" int64_t nvx_moe_order_max_experts(void) { return (48 * 1024 / 4) / 257; }
+
+extern "C" int nvx_moe_order(const int32_t* idx, int64_t n, int64_t n_exp, int64_t* dst, int32_t* counts, nvx_stream_t stream) {
+    NVX_REQUIRE(n >= 0 && n < (1ll << 31) && n_exp > 0 && n_exp <= nvx_moe_order_max_experts(), NVX_EINVAL,
+                "nvx_moe_order: bad sizes (the experts' counters must fit LDS)");
+    NVX_REQUIRE(idx && dst && counts, NVX_EINVAL, "nvx_moe_order: null pointer");
+    hipLaunchKernelGGL(moe_order_kernel, dim3(1), dim3(256), (size_t)(n_exp * 257) * sizeof(int), (hipStream_t)stream, idx, n, (int)n_exp, dst,
+                       counts);
+    return nvx_check_launch("nvx_moe_order");
+}
 
 extern "C" int nvx_moe_route(const float* logits, int64_t n_tok, int64_t n_exp, int64_t top, int32_t* idx, float* wts, nvx_stream_t stream) {
     NVX_REQUIRE(n_tok >= 0 && n_exp > 0 && n_exp < (1 << 20) && top > 0 && top <= n_exp, NVX_EINVAL, "nvx_moe_route: bad sizes");

@@ -15,8 +15,8 @@ class SigmoidInputMoE(nn.Module):
 
     Steps of few tokens (decode steps, which a hipGraph replays: no host decision may depend on the routing) evaluate each
     token's experts in one launch, streaming the chosen experts' rows.  Steps of many tokens put the scaled inputs into
-    expert order and run one pair of matrix products per expert that received tokens; the per-expert counts are the one
-    host read of that path."""
+    expert order (ops.moe_order: a counting sort, which also gives the per-expert counts) and run one pair of matrix
+    products per expert that received tokens; the counts are the one host read of that path."""
 
     ROWS_PATH_TOKENS = 32
 
@@ -35,12 +35,16 @@ class SigmoidInputMoE(nn.Module):
             self._rows_fit = ops.moe_expert_rows_fits(self.width, self.ff)
         if self._rows_fit and (decode_step or t <= self.ROWS_PATH_TOKENS):
             return ops.moe_expert_rows(h, idx, wts, self.w_gu, self.w_d, self.limit, self.alpha)
-        flat = idx.view(-1).long()
-        order = torch.argsort(flat, stable=True)
-        dst = torch.empty_like(order)
-        dst[order] = torch.arange(order.numel(), device=order.device)
-        dst = dst.view(t, self.top)
-        counts = torch.bincount(flat, minlength=self.experts).tolist()
+        if ops.moe_order_fits(self.experts):
+            dst, counts = ops.moe_order(idx, self.experts)
+            counts = counts.tolist()
+        else:                                  # more experts than the ordering kernel's counters hold: a library sort
+            flat = idx.view(-1).long()
+            order = torch.argsort(flat, stable=True)
+            dst = torch.empty_like(order)
+            dst[order] = torch.arange(order.numel(), device=order.device)
+            dst = dst.view(t, self.top)
+            counts = torch.bincount(flat, minlength=self.experts).tolist()
         xs = ops.moe_scatter_rows(h, wts, dst)
         gu = torch.empty((xs.shape[0], 2 * self.ff), dtype=h.dtype, device=h.device)
         a = 0

@@ -1111,6 +1111,22 @@ def moe_expert_rows(h, idx, wts, w_gu, w_d, limit: float, alpha: float):
     return out
 
 
+def moe_order_fits(n_exp: int) -> bool:
+    return n_exp <= _lib.load().nvx_moe_order_max_experts()
+
+
+def moe_order(idx, n_exp: int):
+    """idx (T, top) int32 expert ids -> (dst (T, top) int64, counts (n_exp) int32): dst[t][k] is the place of pair (t, k) when all
+    pairs are put in expert order (pairs of one expert keep their order), counts[e] the pairs of expert e."""
+    _dev(idx)
+    _need(idx.dtype == torch.int32 and idx.is_contiguous() and idx.dim() == 2, "moe_order: idx must be contiguous int32 (T, top)")
+    dst = torch.empty(idx.shape, dtype=torch.int64, device=idx.device)
+    counts = torch.empty((n_exp,), dtype=torch.int32, device=idx.device)
+    lib = _lib.load()
+    _lib.check(lib.nvx_moe_order(_ptr(idx), idx.numel(), n_exp, _ptr(dst), _ptr(counts), _stream()), "nvx_moe_order")
+    return dst, counts
+
+
 def moe_scatter_rows(h, wts, dst):
     """xs[dst[r]] = wts[r] * h[r // top] for every (token, choice) pair r (dst: int64 (T, top), a permutation)."""
     _dev(h, wts, dst)

@@ -86,6 +86,7 @@ _DEFS = {
                     "Tensor state_slot, Tensor? qo_indptr, Tensor? tok_seq, float scale, float cap, int heads, int kv_heads, int dim, int vdim) -> Tensor",
     "moe_route": "(Tensor logits, int top) -> (Tensor, Tensor)",
     "moe_expert_rows": "(Tensor h, Tensor idx, Tensor wts, Tensor w_gu, Tensor w_d, float limit, float alpha) -> Tensor",
+    "moe_order": "(Tensor idx, int n_exp) -> (Tensor, Tensor)",
     "moe_scatter_rows": "(Tensor h, Tensor wts, Tensor dst) -> Tensor",
     "moe_glu": "(Tensor gu, float limit, float alpha) -> Tensor",
     "moe_gather_rows": "(Tensor ys, Tensor dst) -> Tensor",
@@ -294,6 +295,10 @@ def _moe_route(logits, top):
 
 def _moe_expert_rows(h, idx, wts, w_gu, w_d, limit, alpha):
     return ops.moe_expert_rows(h, idx, wts, w_gu, w_d, limit, alpha)
+
+
+def _moe_order(idx, n_exp):
+    return ops.moe_order(idx, n_exp)
 
 
 def _moe_scatter_rows(h, wts, dst):

@@ -286,6 +286,20 @@ def test_capped_attention_finds_one_key_among_hundreds(fmt, vdim):
     assert (out[1, 3] - out[2, 3]).abs().max() > 0.1          # the last query's own key changes head 3
 
 
+@pytest.mark.parametrize("n_tok,top,experts", [(20000, 2, 8), (5, 1, 1), (300, 3, 47), (257, 1, 2)])
+def test_expert_order_is_a_stable_counting_sort(n_tok, top, experts):
+    from nano_vllm_x_amd import ops
+    g = torch.Generator().manual_seed(n_tok)
+    idx = torch.randint(0, experts, (n_tok, top), generator=g, dtype=torch.int32)
+    dst, counts = ops.moe_order(idx.cuda(), experts)
+    flat = idx.view(-1).long()
+    order = torch.sort(flat, stable=True).indices          # on the host
+    want = torch.empty_like(order)
+    want[order] = torch.arange(order.numel())
+    assert torch.equal(dst.cpu().view(-1), want) and torch.equal(counts.cpu().long(), torch.bincount(flat, minlength=experts))
+    assert ops.moe_order_fits(47) and not ops.moe_order_fits(4000)
+
+
 @pytest.mark.parametrize("top,experts", [(1, 1), (1, 4), (2, 5), (3, 3)])
 def test_experts_by_rows_and_by_expert_order_agree_with_the_restatement(top, experts):
     from nano_vllm_x_amd.layers.moe import SigmoidInputMoE
