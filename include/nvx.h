@@ -44,7 +44,7 @@ typedef void* nvx_stream_t;
  *   8: layers with a 32-bit residual stream and per-sequence state (`nvx_boundary_norm`, `nvx_canon_conv`, `nvx_relu2`,
  *      `nvx_mingru_scan`) and latent attention (`nvx_latent_prep`, `nvx_latent_attn`) added.
  *   9: nvx_boundary_norm can apply the convolution of a decode step in the same launch. */
-#define NVX_ABI_VERSION 13
+#define NVX_ABI_VERSION 14
 
 /* Library identification and diagnostics. */
 int nvx_abi_version(void);
@@ -532,8 +532,9 @@ int nvx_latent_attn(const void* q, const void* cache, int fmt, const int32_t* kv
  *     of that logit.
  * Expert e:  g = min(W_gate x, limit), u = clamp(W_up x, -limit, limit), y = g sigmoid(alpha g) (u + 1), result W_down y, with
  *     w_gu (experts, 2 ff, width) = rows [gate | up] and w_d (experts, width, ff).
- * nvx_moe_expert_rows:  out[t] = sum_k expert_idx[t][k](wts[t][k] * h[t]), a workgroup per token (width <=
- *     nvx_moe_expert_rows_max_width(ff)).
+ * nvx_moe_expert_rows:  out[t] = sum_k expert_idx[t][k](wts[t][k] * h[t]), the experts' rows streamed per (token, choice) pair by
+ *     workgroups of 64 rows; ws: n_tok * top * ff floats (the hidden activations between its two launches); width <=
+ *     nvx_moe_expert_rows_max_width(ff).
  * nvx_moe_order:  dst[r] = place of pair r (= token * top + choice) when the n pairs are put in expert order, pairs of one expert
  *     keeping their order; counts[e] = pairs of expert e.  n_exp <= nvx_moe_order_max_experts().
  * nvx_moe_scatter_rows:  xs[dst[r]] = wts[r] * h[r / top] for every (token, choice) pair r.
@@ -579,8 +580,8 @@ int nvx_softcap_attn(const void* q, const void* k_cache, const void* v_cache, in
 int nvx_moe_route(const float* logits, int64_t n_tok, int64_t n_exp, int64_t top, int32_t* idx, float* wts, nvx_stream_t stream);
 int64_t nvx_moe_expert_rows_max_width(int64_t ff);
 int nvx_moe_expert_rows(const void* h, int64_t h_stride, int fmt, const int32_t* idx, const float* wts, int64_t top,
-                        const void* w_gu, const void* w_d, int64_t n_exp, float limit, float alpha, void* out, int64_t n_tok,
-                        int64_t width, int64_t ff, nvx_stream_t stream);
+                        const void* w_gu, const void* w_d, int64_t n_exp, float limit, float alpha, float* ws, void* out,
+                        int64_t n_tok, int64_t width, int64_t ff, nvx_stream_t stream);
 int64_t nvx_moe_order_max_experts(void);
 int nvx_moe_order(const int32_t* idx, int64_t n, int64_t n_exp, int64_t* dst, int32_t* counts, nvx_stream_t stream);
 int nvx_moe_scatter_rows(const void* h, int64_t h_stride, int fmt, const float* wts, const int64_t* dst, int64_t top, void* xs,

@@ -1,7 +1,7 @@
 // Mixture of small gated feed-forward experts with a sigmoid router whose weight scales the chosen expert's INPUT.
 //   - nvx_moe_route: the `top` largest router logits of every token -> expert ids and sigmoid scores (float32);
-//   - nvx_moe_expert_rows: a token's experts evaluated row by row of their weights (a workgroup per token): the form for
-//     steps of few tokens, where every chosen expert's weights have to be streamed once per token anyway;
+//   - nvx_moe_expert_rows: a token's experts evaluated row by row of their weights: the form for steps of few tokens, where
+//     every chosen expert's weights have to be streamed once per token anyway;
 //   - nvx_moe_order / nvx_moe_scatter_rows / nvx_moe_glu / nvx_moe_gather_rows: the pieces around per-expert matrix products
 //     for steps of many tokens (the expert order of the (token, choice) pairs and the experts' counts, scaled inputs gathered
 //     into that order, the gated activation, the tokens' results summed back).
@@ -34,51 +34,75 @@ __device__ __forceinline__ float glu_act(float g, float u, float limit, float al
     return g * sigmoid_f(alpha * g) * (u + 1.0f);
 }
 
-// w_gu: (experts, 2 * ff, width) rows [gate | up]; w_d: (experts, width, ff).  LDS: the scaled input (width), the hidden
-// activations (ff), the running output (width).
-template <typename A>
-__global__ __launch_bounds__(256) void moe_expert_rows_kernel(const A* __restrict__ h, int64_t h_stride, const int32_t* __restrict__ idx,
-                                                             const float* __restrict__ wts, int top, const A* __restrict__ w_gu,
-                                                             const A* __restrict__ w_d, float limit, float alpha, A* __restrict__ out,
-                                                             int width, int ff) {
-    extern __shared__ float sm[];
-    float* xs = sm;
-    float* ys = xs + width;
-    float* os = ys + ff;
-    const int64_t t = blockIdx.x;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    for (int k = 0; k < top; ++k) {
-        const int e = idx[t * top + k];
-        const float wt = wts[t * top + k];
-        __syncthreads();
-        for (int c = threadIdx.x; c < width; c += 256) xs[c] = (float)(A)(wt * ld_f(h, t * h_stride + c));
-        __syncthreads();
-        const A* wg = w_gu + (int64_t)e * 2 * ff * width;
-        for (int j = wave; j < ff; j += 4) {
-            const A* gr = wg + (int64_t)j * width;
-            const A* ur = wg + (int64_t)(ff + j) * width;
-            float g = 0.f, u = 0.f;
-            for (int c = lane; c < width; c += 64) {
-                const float x = xs[c];
-                g += ld_f(gr, c) * x;
-                u += ld_f(ur, c) * x;
-            }
-            g = wave_sum(g);
-            u = wave_sum(u);
-            if (lane == 0) ys[j] = (float)(A)glu_act((float)(A)g, (float)(A)u, limit, alpha);
+// A token's experts row by row.  w_gu: (experts, 2 * ff, width) rows [gate | up]; w_d: (experts, width, ff).  Two launches, both
+// with a workgroup per 64 weight rows so that a step of a few tokens still fills the chip: the hidden activations of every
+// (token, choice) pair into a float32 workspace, then the output rows summed over a token's choices.  A wave takes 16 rows; its
+// lanes walk a row 8 elements at a time (16-byte loads) where the format is 16-bit and the rows are 16-byte aligned.
+template <typename A, bool VEC>
+__device__ __forceinline__ float lane_dot(const A* __restrict__ wrow, const float* __restrict__ xs, int n, int lane) {
+    float acc = 0.f;
+    if constexpr (VEC) {
+        typedef A vec8 __attribute__((ext_vector_type(8)));
+        for (int c = lane * 8; c < n; c += 512) {
+            const vec8 v = *reinterpret_cast<const vec8*>(wrow + c);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc += (float)v[i] * xs[c + i];
         }
+    } else {
+        for (int c = lane; c < n; c += 64) acc += ld_f(wrow, c) * xs[c];
+    }
+    return acc;
+}
+
+constexpr int MOE_ROWS = 64;      // weight rows per workgroup (16 per wave)
+
+template <typename A, bool VEC>
+__global__ __launch_bounds__(256) void moe_rows_up_kernel(const A* __restrict__ h, int64_t h_stride, const int32_t* __restrict__ idx,
+                                                         const float* __restrict__ wts, int top, const A* __restrict__ w_gu, float limit,
+                                                         float alpha, float* __restrict__ y, int width, int ff) {
+    extern __shared__ float sm[];      // the scaled input (width)
+    const int64_t t = blockIdx.z;
+    const int k = blockIdx.y;
+    const int e = idx[t * top + k];
+    const float wt = wts[t * top + k];
+    for (int c = threadIdx.x; c < width; c += 256) sm[c] = (float)(A)(wt * ld_f(h, t * h_stride + c));
+    __syncthreads();
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const A* wg = w_gu + (int64_t)e * 2 * ff * width;
+    for (int i = 0; i < MOE_ROWS / 4; ++i) {
+        const int j = blockIdx.x * MOE_ROWS + wave * (MOE_ROWS / 4) + i;
+        if (j >= ff) break;
+        const float g = wave_sum(lane_dot<A, VEC>(wg + (int64_t)j * width, sm, width, lane));
+        const float u = wave_sum(lane_dot<A, VEC>(wg + (int64_t)(ff + j) * width, sm, width, lane));
+        if (lane == 0) y[(t * top + k) * ff + j] = (float)(A)glu_act((float)(A)g, (float)(A)u, limit, alpha);
+    }
+}
+
+template <typename A, bool VEC>
+__global__ __launch_bounds__(256) void moe_rows_down_kernel(const float* __restrict__ y, const int32_t* __restrict__ idx, int top,
+                                                           const A* __restrict__ w_d, A* __restrict__ out, int width, int ff) {
+    extern __shared__ float sm[];      // one choice's hidden activations (ff)
+    const int64_t t = blockIdx.y;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    float o[MOE_ROWS / 4];
+#pragma unroll
+    for (int i = 0; i < MOE_ROWS / 4; ++i) o[i] = 0.f;
+    for (int k = 0; k < top; ++k) {
         __syncthreads();
-        const A* wd = w_d + (int64_t)e * width * ff;
-        for (int c = wave; c < width; c += 4) {
-            const A* dr = wd + (int64_t)c * ff;
-            float o = 0.f;
-            for (int j = lane; j < ff; j += 64) o += ld_f(dr, j) * ys[j];
-            o = wave_sum(o);
-            if (lane == 0) os[c] = (k ? os[c] : 0.f) + (float)(A)o;
+        for (int j = threadIdx.x; j < ff; j += 256) sm[j] = y[(t * top + k) * ff + j];
+        __syncthreads();
+        const A* wd = w_d + (int64_t)idx[t * top + k] * width * ff;
+#pragma unroll
+        for (int i = 0; i < MOE_ROWS / 4; ++i) {
+            const int c = blockIdx.x * MOE_ROWS + wave * (MOE_ROWS / 4) + i;
+            if (c < width) o[i] += (float)(A)wave_sum(lane_dot<A, VEC>(wd + (int64_t)c * ff, sm, ff, lane));
         }
     }
-    __syncthreads();
-    for (int c = threadIdx.x; c < width; c += 256) st_f(out, t * (int64_t)width + c, os[c]);
+#pragma unroll
+    for (int i = 0; i < MOE_ROWS / 4; ++i) {
+        const int c = blockIdx.x * MOE_ROWS + wave * (MOE_ROWS / 4) + i;
+        if (c < width && lane == 0) st_f(out, t * (int64_t)width + c, o[i]);
+    }
 }
 
 // xs[dst[r]] = wts[r] * h[r / top]  for every (token, choice) pair r: the experts' inputs in expert order
@@ -175,22 +199,39 @@ extern "C" int nvx_moe_route(const float* logits, int64_t n_tok, int64_t n_exp, 
 }
 
 extern "C" int64_t nvx_moe_expert_rows_max_width(int64_t ff) {
-    const int64_t room = 65536 / 4 - ff;          // floats of the default LDS window left for the input and the output
-    return room > 0 ? room / 2 : 0;
+    return ff > 0 && ff <= 12288 ? 12288 : 0;      // a row of either size waits in LDS as float32
+}
+
+template <typename A>
+static void launch_moe_rows(const void* h, int64_t h_stride, const int32_t* idx, const float* wts, int top, const void* w_gu, const void* w_d,
+                            float limit, float alpha, float* ws, void* out, int64_t n_tok, int width, int ff, hipStream_t s) {
+    const bool vec = sizeof(A) == 2 && width % 8 == 0 && ff % 8 == 0 && nvx_aligned16(w_gu) && nvx_aligned16(w_d);
+    const dim3 up((unsigned)((ff + MOE_ROWS - 1) / MOE_ROWS), (unsigned)top, (unsigned)n_tok);
+    const dim3 down((unsigned)((width + MOE_ROWS - 1) / MOE_ROWS), (unsigned)n_tok);
+    if (vec) {
+        hipLaunchKernelGGL((moe_rows_up_kernel<A, true>), up, dim3(256), (size_t)width * sizeof(float), s, (const A*)h, h_stride, idx, wts, top,
+                           (const A*)w_gu, limit, alpha, ws, width, ff);
+        hipLaunchKernelGGL((moe_rows_down_kernel<A, true>), down, dim3(256), (size_t)ff * sizeof(float), s, (const float*)ws, idx, top,
+                           (const A*)w_d, (A*)out, width, ff);
+    } else {
+        hipLaunchKernelGGL((moe_rows_up_kernel<A, false>), up, dim3(256), (size_t)width * sizeof(float), s, (const A*)h, h_stride, idx, wts, top,
+                           (const A*)w_gu, limit, alpha, ws, width, ff);
+        hipLaunchKernelGGL((moe_rows_down_kernel<A, false>), down, dim3(256), (size_t)ff * sizeof(float), s, (const float*)ws, idx, top,
+                           (const A*)w_d, (A*)out, width, ff);
+    }
 }
 
 extern "C" int nvx_moe_expert_rows(const void* h, int64_t h_stride, int fmt, const int32_t* idx, const float* wts, int64_t top,
-                                   const void* w_gu, const void* w_d, int64_t n_exp, float limit, float alpha, void* out, int64_t n_tok,
-                                   int64_t width, int64_t ff, nvx_stream_t stream) {
+                                   const void* w_gu, const void* w_d, int64_t n_exp, float limit, float alpha, float* ws, void* out,
+                                   int64_t n_tok, int64_t width, int64_t ff, nvx_stream_t stream) {
     NVX_REQUIRE(fmt >= 0 && fmt <= 2, NVX_EINVAL, "nvx_moe_expert_rows: fmt must be 0, 1 or 2");
-    NVX_REQUIRE(n_tok >= 0 && top > 0 && n_exp > 0 && width > 0 && ff > 0 && h_stride >= width, NVX_EINVAL, "nvx_moe_expert_rows: bad sizes");
-    NVX_REQUIRE(width <= nvx_moe_expert_rows_max_width(ff), NVX_EUNSUPPORTED, "nvx_moe_expert_rows: a row and the hidden size do not fit LDS");
+    NVX_REQUIRE(n_tok >= 0 && n_tok <= 65535 && top > 0 && top <= 65535 && n_exp > 0 && width > 0 && ff > 0 && h_stride >= width, NVX_EINVAL,
+                "nvx_moe_expert_rows: bad sizes (at most 65535 tokens a step)");
+    NVX_REQUIRE(width <= nvx_moe_expert_rows_max_width(ff), NVX_EUNSUPPORTED, "nvx_moe_expert_rows: a row or the hidden size does not fit LDS");
     if (n_tok == 0) return NVX_OK;
-    NVX_REQUIRE(h && idx && wts && w_gu && w_d && out, NVX_EINVAL, "nvx_moe_expert_rows: null pointer");
-    const size_t lds = (size_t)(2 * width + ff) * sizeof(float);
-    NVX_FMT_CALL(fmt, hipLaunchKernelGGL(moe_expert_rows_kernel<A_>, dim3((unsigned)n_tok), dim3(256), lds, (hipStream_t)stream, (const A_*)h,
-                                         h_stride, idx, wts, (int)top, (const A_*)w_gu, (const A_*)w_d, limit, alpha, (A_*)out, (int)width,
-                                         (int)ff));
+    NVX_REQUIRE(h && idx && wts && w_gu && w_d && ws && out, NVX_EINVAL, "nvx_moe_expert_rows: null pointer");
+    NVX_FMT_CALL(fmt, launch_moe_rows<A_>(h, h_stride, idx, wts, (int)top, w_gu, w_d, limit, alpha, ws, out, n_tok, (int)width, (int)ff,
+                                          (hipStream_t)stream));
     return nvx_check_launch("nvx_moe_expert_rows");
 }
 

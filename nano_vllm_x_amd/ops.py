@@ -1098,16 +1098,17 @@ def _moe_weights(w_gu, w_d, what: str):
 
 def moe_expert_rows(h, idx, wts, w_gu, w_d, limit: float, alpha: float):
     """out[t] = sum over token t's chosen experts of expert(score * h[t]); w_gu (experts, 2 * ff, width) = gate | up rows, w_d
-    (experts, width, ff).  One workgroup per token: the form for steps of few tokens."""
+    (experts, width, ff).  The chosen experts' rows are streamed per (token, choice) pair: the form for steps of few tokens."""
     _dev(h, idx, wts, w_gu, w_d)
     n_exp, ff, width = _moe_weights(w_gu, w_d, "moe_expert_rows")
     t, top = idx.shape
     _need(h.shape == (t, width) and h.stride(1) == 1 and h.dtype == w_gu.dtype, "moe_expert_rows: h shape / format")
     _need(idx.dtype == torch.int32 and idx.is_contiguous() and wts.dtype == F32 and wts.is_contiguous() and wts.shape == idx.shape, "moe_expert_rows: choices")
     out = torch.empty((t, width), dtype=h.dtype, device=h.device)
+    ws = torch.empty((t, top, ff), dtype=F32, device=h.device)      # the hidden activations between the two launches
     lib = _lib.load()
     _lib.check(lib.nvx_moe_expert_rows(_ptr(h), h.stride(0), _fmt(h), _ptr(idx), _ptr(wts), top, _ptr(w_gu), _ptr(w_d), n_exp, float(limit),
-                                       float(alpha), _ptr(out), t, width, ff, _stream()), "nvx_moe_expert_rows")
+                                       float(alpha), _ptr(ws), _ptr(out), t, width, ff, _stream()), "nvx_moe_expert_rows")
     return out
 
 
