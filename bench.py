@@ -516,7 +516,7 @@ def _meronex_config(z):
             "layers": [(par, mls, dlt)[i % 3] for i in range(z["layers"])]}
 
 
-def _meronex_kernel_table(z, t_pre, n_dec, ctx):
+def _meronex_kernel_table(z, t_pre, n_dec, ctx, phases=("prefill", "decode")):
     """Each kernel of Meronex beside the like kernel of Qwen3 (or of the other seq-state model) at the same shape: time, and the
     fraction of its roofline (HBM bytes it must move at 8 TB/s; attention in prefill: its multiply-adds at the dense bf16 MFMA
     peak; the recurrences in prefill: their multiply-adds at the float32 vector peak, since their state is float32)."""
@@ -542,6 +542,8 @@ def _meronex_kernel_table(z, t_pre, n_dec, ctx):
         rows.append({"kernel": name, "phase": phase, "us": round(us, 1), "of_roofline": round(frac, 3), "bound": bound, "like": like})
 
     for phase, (n_seq, q_len, pos0) in (("prefill", (t_pre // 1024, 1024, 0)), ("decode", (n_dec, 1, ctx))):
+        if phase not in phases:
+            continue
         t = n_seq * q_len
         lay = layout(n_seq, q_len, pos0)
         reps = 3 if phase == "prefill" else 20
@@ -641,8 +643,8 @@ def _meronex_kernel_table(z, t_pre, n_dec, ctx):
     return rows
 
 
-ARCHS = {"kabidra": (lambda z: _kabidra_config(z), lambda *a: _kernel_table(*a), "Kabidra"),
-         "meronex": (lambda z: _meronex_config(z), lambda *a: _meronex_kernel_table(*a), "Meronex")}
+ARCHS = {"kabidra": (lambda z: _kabidra_config(z), lambda *a, **k: _kernel_table(*a), "Kabidra"),
+         "meronex": (lambda z: _meronex_config(z), lambda *a, **k: _meronex_kernel_table(*a, **k), "Meronex")}
 
 
 def arch_compare(args):
@@ -676,7 +678,8 @@ def arch_compare(args):
             continue
         print(f"[arch-compare] {name}: kernels one by one", file=sys.stderr, flush=True)
         with torch.inference_mode():
-            entry["kernels"] = kernel_table(z, args.arch_seqs * args.arch_prompt, args.arch_seqs, args.arch_prompt)
+            entry["kernels"] = kernel_table(z, args.arch_seqs * args.arch_prompt, args.arch_seqs, args.arch_prompt,
+                                            phases=tuple(args.arch_phases.split(",")))
         result["sizes"][name] = entry
     print(json.dumps(result), flush=True)
 
@@ -688,6 +691,7 @@ def main():
                          "each of its kernels beside the like Qwen3 kernel against its roofline (one JSON line)")
     ap.add_argument("--arch", choices=sorted(ARCHS), default="kabidra", help="the design that --arch-compare puts beside Qwen3")
     ap.add_argument("--arch-portion", type=int, default=0, help="--arch-compare: compute the prompts in steps of at most this many tokens")
+    ap.add_argument("--arch-phases", default="prefill,decode", help="--arch-compare --arch meronex: which shapes the kernels one by one run at")
     ap.add_argument("--arch-serve", type=int, default=1, help="--arch-compare: 0 skips the engines (kernels one by one only)")
     ap.add_argument("--arch-kernels", type=int, default=1, help="--arch-compare: 0 skips the kernels one by one (engines only)")
     ap.add_argument("--arch-sizes", default="w1024,w2048,w4096")

@@ -533,7 +533,7 @@ int nvx_latent_attn(const void* q, const void* cache, int fmt, const int32_t* kv
  * Expert e:  g = min(W_gate x, limit), u = clamp(W_up x, -limit, limit), y = g sigmoid(alpha g) (u + 1), result W_down y, with
  *     w_gu (experts, 2 ff, width) = rows [gate | up] and w_d (experts, width, ff).
  * nvx_moe_expert_rows:  out[t] = sum_k expert_idx[t][k](wts[t][k] * h[t]), the experts' rows streamed per (token, choice) pair by
- *     workgroups of 64 rows; ws: n_tok * top * ff floats (the hidden activations between its two launches); width <=
+ *     workgroups of a few dozen rows; ws: n_tok * top * ff floats (the hidden activations between its two launches); width <=
  *     nvx_moe_expert_rows_max_width(ff).
  * nvx_moe_order:  dst[r] = place of pair r (= token * top + choice) when the n pairs are put in expert order, pairs of one expert
  *     keeping their order; counts[e] = pairs of expert e.  n_exp <= nvx_moe_order_max_experts().

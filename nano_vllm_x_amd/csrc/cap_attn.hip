@@ -57,12 +57,12 @@ __device__ __forceinline__ float lane_value(float v, int lane) {      // `lane` 
 // One workgroup of four waves per (head, token).  The waves take the visible keys in tiles of 64, every fourth tile each: a
 // lane scores one key (the query waits in LDS), the wave keeps a running maximum and sum, then each lane accumulates the
 // weighted values of EPL of the head's value columns over the tile's keys.  The four partial results are merged through LDS.
-template <typename A, int EPL>
+template <typename A, int EPL, bool VEC>
 __global__ __launch_bounds__(256) void softcap_attn_kernel(const A* __restrict__ q, const A* __restrict__ k_cache, const A* __restrict__ v_cache,
                                                           const int32_t* __restrict__ kv_indices, const int64_t* __restrict__ kv_start,
                                                           const int32_t* __restrict__ kv_len, const int32_t* __restrict__ qo_indptr,
                                                           const int32_t* __restrict__ tok_seq, float scale, float cap, A* __restrict__ out,
-                                                          int heads, int kv_heads, int dim, int vdim) {
+                                                          int heads, int kv_heads, int dim, int vdim, int vec_v_ok) {
     extern __shared__ float sm[];
     float* sq = sm;                   // dim
     float* sacc = sq + dim;           // 4 * vdim
@@ -83,6 +83,9 @@ __global__ __launch_bounds__(256) void softcap_attn_kernel(const A* __restrict__
     float acc[EPL];
 #pragma unroll
     for (int c = 0; c < EPL; ++c) acc[c] = 0.f;
+    float acc8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    // value rows by 16-byte loads: vdim = 8 * (a power of two up to 64), rows 16-byte aligned (the caller checks the base)
+    const bool vec_values = VEC && (vdim & 7) == 0 && ((vdim >> 3) & ((vdim >> 3) - 1)) == 0 && (vdim >> 3) <= 64 && vec_v_ok;
     for (int j0 = wave * 64; j0 < visible; j0 += 256) {
         const int j = j0 + lane;
         const bool valid = j < visible;
@@ -91,7 +94,16 @@ __global__ __launch_bounds__(256) void softcap_attn_kernel(const A* __restrict__
         if (valid) {
             const A* kr = k_cache + slot * k_row + (int64_t)kvh * dim;
             float dot = 0.f;
-            for (int d = 0; d < dim; ++d) dot += sq[d] * ld_f(kr, d);
+            if constexpr (VEC) {          // 16-bit rows, 16-byte aligned, dim a multiple of 8: eight elements a load
+                typedef A vec8 __attribute__((ext_vector_type(8)));
+                for (int d = 0; d < dim; d += 8) {
+                    const vec8 kv = *reinterpret_cast<const vec8*>(kr + d);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) dot += sq[d + i] * (float)kv[i];
+                }
+            } else {
+                for (int d = 0; d < dim; ++d) dot += sq[d] * ld_f(kr, d);
+            }
             s = dot * scale;
             if (cap > 0.f) s = cap * tanhf(s / cap);
         }
@@ -103,6 +115,27 @@ __global__ __launch_bounds__(256) void softcap_attn_kernel(const A* __restrict__
 #pragma unroll
         for (int c = 0; c < EPL; ++c) acc[c] *= corr;
         const int n_here = visible - j0 < 64 ? visible - j0 : 64;
+        if constexpr (VEC) {
+            // a value row is vdim / 8 lanes of eight elements (16-byte loads), so 64 / (vdim / 8) keys are taken at a time
+            if (vec_values) {
+                const int lpr = vdim >> 3, grp = lane / lpr, groups = 64 / lpr;
+                typedef A vec8 __attribute__((ext_vector_type(8)));
+#pragma unroll
+                for (int i = 0; i < 8; ++i) acc8[i] *= corr;
+                for (int j1 = 0; j1 < n_here; j1 += groups) {
+                    const int jj = j1 + grp;
+                    const int src = jj < n_here ? jj : 0;
+                    const float pj = __shfl(p, src, 64);
+                    const int sl = __shfl(slot, src, 64);
+                    if (jj < n_here) {
+                        const vec8 vv = *reinterpret_cast<const vec8*>(v_cache + sl * v_row + (int64_t)kvh * vdim + (lane % lpr) * 8);
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) acc8[i] += pj * (float)vv[i];
+                    }
+                }
+                continue;
+            }
+        }
         for (int jj = 0; jj < n_here; ++jj) {
             const float pj = lane_value(p, jj);
             const int sl = __builtin_amdgcn_readlane(slot, jj);
@@ -114,10 +147,22 @@ __global__ __launch_bounds__(256) void softcap_attn_kernel(const A* __restrict__
             }
         }
     }
+    if (VEC && vec_values) {
+        const int lpr = vdim >> 3;
+        for (int mk = lpr; mk < 64; mk <<= 1) {
 #pragma unroll
-    for (int c = 0; c < EPL; ++c) {
-        const int e = lane + 64 * c;
-        if (e < vdim) sacc[wave * vdim + e] = acc[c];
+            for (int i = 0; i < 8; ++i) acc8[i] += __shfl_xor(acc8[i], mk, 64);
+        }
+        if (lane < lpr) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) sacc[wave * vdim + lane * 8 + i] = acc8[i];
+        }
+    } else {
+#pragma unroll
+        for (int c = 0; c < EPL; ++c) {
+            const int e = lane + 64 * c;
+            if (e < vdim) sacc[wave * vdim + e] = acc[c];
+        }
     }
     if (lane == 0) { sml[wave] = m; sml[4 + wave] = l; }
     __syncthreads();
@@ -167,14 +212,18 @@ extern "C" int nvx_softcap_attn(const void* q, const void* k_cache, const void* 
     NVX_REQUIRE((tok_seq != nullptr) == (qo_indptr != nullptr), NVX_EINVAL, "nvx_softcap_attn: tok_seq and qo_indptr go together");
     const size_t lds = (size_t)(dim + 4 * vdim + 8) * sizeof(float);
     const dim3 grid((unsigned)heads, (unsigned)n_tok);
-#define NVX_CAP_ATTN(EPL)                                                                                                                 \
-    NVX_FMT_CALL(fmt, hipLaunchKernelGGL((softcap_attn_kernel<A_, EPL>), grid, dim3(256), lds, (hipStream_t)stream, (const A_*)q,          \
-                                         (const A_*)k_cache, (const A_*)v_cache, kv_indices, kv_start, kv_len, qo_indptr, tok_seq, scale,  \
-                                         cap, (A_*)out, (int)heads, (int)kv_heads, (int)dim, (int)vdim))
+#define NVX_CAP_ATTN_V(EPL, VEC)                                                                                                          \
+    NVX_FMT_CALL(fmt, hipLaunchKernelGGL((softcap_attn_kernel<A_, EPL, VEC && sizeof(A_) == 2>), grid, dim3(256), lds, (hipStream_t)stream,     \
+                                         (const A_*)q, (const A_*)k_cache, (const A_*)v_cache, kv_indices, kv_start, kv_len, qo_indptr,      \
+                                         tok_seq, scale, cap, (A_*)out, (int)heads, (int)kv_heads, (int)dim, (int)vdim,       \
+                                         (int)nvx_aligned16(v_cache)))
+#define NVX_CAP_ATTN(EPL) do { if (vec) NVX_CAP_ATTN_V(EPL, true); else NVX_CAP_ATTN_V(EPL, false); } while (0)
+    const bool vec = fmt != 2 && dim % 8 == 0 && nvx_aligned16(k_cache);
     if (vdim <= 64) NVX_CAP_ATTN(1);
     else if (vdim <= 128) NVX_CAP_ATTN(2);
     else if (vdim <= 256) NVX_CAP_ATTN(4);
     else NVX_CAP_ATTN(8);
+#undef NVX_CAP_ATTN_V
 #undef NVX_CAP_ATTN
     return nvx_check_launch("nvx_softcap_attn");
 }

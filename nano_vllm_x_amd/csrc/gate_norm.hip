@@ -90,7 +90,8 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __rest
 // sums have one order, and the launch can be captured.
 template <typename A, int TOK>
 __global__ __launch_bounds__(256) void skinny_proj_kernel(const A* __restrict__ x, int64_t x_stride, const float* __restrict__ w,
-                                                         int in_act, float* __restrict__ out, int64_t n_tok, int n_out, int k_in) {
+                                                         int in_act, float* __restrict__ out, int64_t n_tok, int n_out, int k_in,
+                                                         int out_per_block) {
     extern __shared__ float xs[];      // TOK rows of k_in
     const int64_t t0 = (int64_t)blockIdx.x * TOK;
     const int nt = (int)(n_tok - t0 < TOK ? n_tok - t0 : TOK);
@@ -100,9 +101,11 @@ __global__ __launch_bounds__(256) void skinny_proj_kernel(const A* __restrict__ 
         xs[i] = in_act == 1 ? tanhf(v) : v;
     }
     __syncthreads();
+    const int n_lo = blockIdx.y * out_per_block;
+    const int n_hi = n_lo + out_per_block < n_out ? n_lo + out_per_block : n_out;
     if (k_in >= 256) {
         const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-        for (int n = wave; n < n_out; n += 4) {
+        for (int n = n_lo + wave; n < n_hi; n += 4) {
             const float* wr = w + (int64_t)n * k_in;
             float acc[TOK];
 #pragma unroll
@@ -119,7 +122,7 @@ __global__ __launch_bounds__(256) void skinny_proj_kernel(const A* __restrict__ 
             }
         }
     } else {
-        for (int n = threadIdx.x; n < n_out; n += 256) {
+        for (int n = n_lo + threadIdx.x; n < n_hi; n += 256) {
             const float* wr = w + (int64_t)n * k_in;
             float acc[TOK];
 #pragma unroll
@@ -147,15 +150,22 @@ extern "C" int nvx_skinny_proj(const void* x, int64_t x_stride, int fmt, const f
                 "nvx_skinny_proj: bad sizes (at most 12288 inputs)");
     if (n_tok == 0) return NVX_OK;
     NVX_REQUIRE(x && w && out, NVX_EINVAL, "nvx_skinny_proj: null pointer");
+    // the outputs are split over workgroups too (8 a workgroup for wide inputs, 256 for narrow ones): a step of few tokens would
+    // otherwise be a handful of workgroups walking all outputs one after another
+    const int opb = k_in >= 256 ? 8 : 256;
+    const int64_t chunks = (n_out + opb - 1) / opb;
+    NVX_REQUIRE(chunks <= 65535, NVX_EINVAL, "nvx_skinny_proj: too many outputs");
     if (k_in <= 3072) {
         const int64_t blocks = (n_tok + 3) / 4;
         NVX_REQUIRE(blocks < (1ll << 31), NVX_EINVAL, "nvx_skinny_proj: too many tokens");
-        NVX_FMT_CALL(fmt, hipLaunchKernelGGL((skinny_proj_kernel<A_, 4>), dim3((unsigned)blocks), dim3(256), (size_t)(4 * k_in) * sizeof(float),
-                                             (hipStream_t)stream, (const A_*)x, x_stride, w, in_act, out, n_tok, (int)n_out, (int)k_in));
+        NVX_FMT_CALL(fmt, hipLaunchKernelGGL((skinny_proj_kernel<A_, 4>), dim3((unsigned)blocks, (unsigned)chunks), dim3(256),
+                                             (size_t)(4 * k_in) * sizeof(float), (hipStream_t)stream, (const A_*)x, x_stride, w, in_act, out, n_tok,
+                                             (int)n_out, (int)k_in, opb));
     } else {
         NVX_REQUIRE(n_tok < (1ll << 31), NVX_EINVAL, "nvx_skinny_proj: too many tokens");
-        NVX_FMT_CALL(fmt, hipLaunchKernelGGL((skinny_proj_kernel<A_, 1>), dim3((unsigned)n_tok), dim3(256), (size_t)k_in * sizeof(float),
-                                             (hipStream_t)stream, (const A_*)x, x_stride, w, in_act, out, n_tok, (int)n_out, (int)k_in));
+        NVX_FMT_CALL(fmt, hipLaunchKernelGGL((skinny_proj_kernel<A_, 1>), dim3((unsigned)n_tok, (unsigned)chunks), dim3(256),
+                                             (size_t)k_in * sizeof(float), (hipStream_t)stream, (const A_*)x, x_stride, w, in_act, out, n_tok,
+                                             (int)n_out, (int)k_in, opb));
     }
     return nvx_check_launch("nvx_skinny_proj");
 }

@@ -35,8 +35,8 @@ __device__ __forceinline__ float glu_act(float g, float u, float limit, float al
 }
 
 // A token's experts row by row.  w_gu: (experts, 2 * ff, width) rows [gate | up]; w_d: (experts, width, ff).  Two launches, both
-// with a workgroup per 64 weight rows so that a step of a few tokens still fills the chip: the hidden activations of every
-// (token, choice) pair into a float32 workspace, then the output rows summed over a token's choices.  A wave takes 16 rows; its
+// with a workgroup per 32 weight rows so that a step of a few tokens still fills the chip: the hidden activations of every
+// (token, choice) pair into a float32 workspace, then the output rows summed over a token's choices.  A wave takes 8 rows; its
 // lanes walk a row 8 elements at a time (16-byte loads) where the format is 16-bit and the rows are 16-byte aligned.
 template <typename A, bool VEC>
 __device__ __forceinline__ float lane_dot(const A* __restrict__ wrow, const float* __restrict__ xs, int n, int lane) {
@@ -54,7 +54,7 @@ __device__ __forceinline__ float lane_dot(const A* __restrict__ wrow, const floa
     return acc;
 }
 
-constexpr int MOE_ROWS = 64;      // weight rows per workgroup (16 per wave)
+constexpr int MOE_ROWS = 32;      // weight rows per workgroup (8 per wave)
 
 template <typename A, bool VEC>
 __global__ __launch_bounds__(256) void moe_rows_up_kernel(const A* __restrict__ h, int64_t h_stride, const int32_t* __restrict__ idx,
@@ -69,12 +69,19 @@ __global__ __launch_bounds__(256) void moe_rows_up_kernel(const A* __restrict__ 
     __syncthreads();
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const A* wg = w_gu + (int64_t)e * 2 * ff * width;
+    float g[MOE_ROWS / 4], u[MOE_ROWS / 4];
+#pragma unroll
+    for (int i = 0; i < MOE_ROWS / 4; ++i) {         // all rows' loads in flight before the first reduction
+        const int j = blockIdx.x * MOE_ROWS + wave * (MOE_ROWS / 4) + i;
+        const int jc = j < ff ? j : ff - 1;
+        g[i] = lane_dot<A, VEC>(wg + (int64_t)jc * width, sm, width, lane);
+        u[i] = lane_dot<A, VEC>(wg + (int64_t)(ff + jc) * width, sm, width, lane);
+    }
+#pragma unroll
     for (int i = 0; i < MOE_ROWS / 4; ++i) {
         const int j = blockIdx.x * MOE_ROWS + wave * (MOE_ROWS / 4) + i;
-        if (j >= ff) break;
-        const float g = wave_sum(lane_dot<A, VEC>(wg + (int64_t)j * width, sm, width, lane));
-        const float u = wave_sum(lane_dot<A, VEC>(wg + (int64_t)(ff + j) * width, sm, width, lane));
-        if (lane == 0) y[(t * top + k) * ff + j] = (float)(A)glu_act((float)(A)g, (float)(A)u, limit, alpha);
+        const float gs = wave_sum(g[i]), us = wave_sum(u[i]);
+        if (lane == 0 && j < ff) y[(t * top + k) * ff + j] = (float)(A)glu_act((float)(A)gs, (float)(A)us, limit, alpha);
     }
 }
 
@@ -92,11 +99,14 @@ __global__ __launch_bounds__(256) void moe_rows_down_kernel(const float* __restr
         for (int j = threadIdx.x; j < ff; j += 256) sm[j] = y[(t * top + k) * ff + j];
         __syncthreads();
         const A* wd = w_d + (int64_t)idx[t * top + k] * width * ff;
+        float part[MOE_ROWS / 4];
 #pragma unroll
         for (int i = 0; i < MOE_ROWS / 4; ++i) {
             const int c = blockIdx.x * MOE_ROWS + wave * (MOE_ROWS / 4) + i;
-            if (c < width) o[i] += (float)(A)wave_sum(lane_dot<A, VEC>(wd + (int64_t)c * ff, sm, ff, lane));
+            part[i] = lane_dot<A, VEC>(wd + (int64_t)(c < width ? c : width - 1) * ff, sm, ff, lane);
         }
+#pragma unroll
+        for (int i = 0; i < MOE_ROWS / 4; ++i) o[i] += (float)(A)wave_sum(part[i]);
     }
 #pragma unroll
     for (int i = 0; i < MOE_ROWS / 4; ++i) {

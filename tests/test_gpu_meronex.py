@@ -252,7 +252,7 @@ def test_rotation_with_stretched_frequencies():
 
 
 @pytest.mark.parametrize("fmt", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("vdim", [10, 100, 200, 300])
+@pytest.mark.parametrize("vdim", [8, 10, 64, 100, 128, 200, 300, 512])
 def test_capped_attention_finds_one_key_among_hundreds(fmt, vdim):
     """Keys scattered over the pool in a shuffled order; one key far back carries a score that stands out only through the
     cap's shape (its raw score is far above the cap, the others' are small), so the read-out is that key's value unless a
