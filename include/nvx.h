@@ -44,7 +44,7 @@ typedef void* nvx_stream_t;
  *   8: layers with a 32-bit residual stream and per-sequence state (`nvx_boundary_norm`, `nvx_canon_conv`, `nvx_relu2`,
  *      `nvx_mingru_scan`) and latent attention (`nvx_latent_prep`, `nvx_latent_attn`) added.
  *   9: nvx_boundary_norm can apply the convolution of a decode step in the same launch. */
-#define NVX_ABI_VERSION 15
+#define NVX_ABI_VERSION 14
 
 /* Library identification and diagnostics. */
 int nvx_abi_version(void);
@@ -536,11 +536,7 @@ int nvx_latent_attn(const void* q, const void* cache, int fmt, const int32_t* kv
  *     workgroups of a few dozen rows; ws: n_tok * top * ff floats (the hidden activations between its two launches); width <=
  *     nvx_moe_expert_rows_max_width(ff).
  * nvx_moe_order:  dst[r] = place of pair r (= token * top + choice) when the n pairs are put in expert order, pairs of one expert
- *     keeping their order; counts[e] = pairs of expert e; optionally order[place] = r (the inverse of dst) and offsets[e] = first
- *     place of expert e (n_exp + 1 entries).  n_exp <= nvx_moe_order_max_experts().
- * nvx_moe_expert_grouped:  out_pairs[place] = expert_e(wts[r] * h[r / top]) for every pair r = order[place] of every expert e
- *     (places offsets[e] .. offsets[e + 1]), an expert's weights read once for up to four of its pairs; ws: n_tok * top * ff floats;
- *     width, ff <= nvx_moe_expert_grouped_max_width().  nvx_moe_gather_rows(out_pairs, dst) then sums a token's choices.
+ *     keeping their order; counts[e] = pairs of expert e.  n_exp <= nvx_moe_order_max_experts().
  * nvx_moe_scatter_rows:  xs[dst[r]] = wts[r] * h[r / top] for every (token, choice) pair r.
  * nvx_moe_glu:  y[r][j] = the expert's activation of (gu[r][j], gu[r][ff + j]).
  * nvx_moe_gather_rows:  out[t] = sum_k ys[dst[t * top + k]].
@@ -587,12 +583,7 @@ int nvx_moe_expert_rows(const void* h, int64_t h_stride, int fmt, const int32_t*
                         const void* w_gu, const void* w_d, int64_t n_exp, float limit, float alpha, float* ws, void* out,
                         int64_t n_tok, int64_t width, int64_t ff, nvx_stream_t stream);
 int64_t nvx_moe_order_max_experts(void);
-int nvx_moe_order(const int32_t* idx, int64_t n, int64_t n_exp, int64_t* dst, int32_t* counts, int32_t* order, int32_t* offsets,
-                  nvx_stream_t stream);
-int64_t nvx_moe_expert_grouped_max_width(void);
-int nvx_moe_expert_grouped(const void* h, int64_t h_stride, int fmt, const float* wts, int64_t top, const int32_t* order,
-                           const int32_t* offsets, const void* w_gu, const void* w_d, int64_t n_exp, float limit, float alpha,
-                           float* ws, void* out_pairs, int64_t n_tok, int64_t width, int64_t ff, nvx_stream_t stream);
+int nvx_moe_order(const int32_t* idx, int64_t n, int64_t n_exp, int64_t* dst, int32_t* counts, nvx_stream_t stream);
 int nvx_moe_scatter_rows(const void* h, int64_t h_stride, int fmt, const float* wts, const int64_t* dst, int64_t top, void* xs,
                          int64_t n_tok, int64_t width, nvx_stream_t stream);
 int nvx_moe_glu(const void* gu, int fmt, float limit, float alpha, void* y, int64_t rows, int64_t ff, nvx_stream_t stream);

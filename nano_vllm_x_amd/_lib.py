@@ -115,10 +115,7 @@ SIGNATURES = {
     "nvx_moe_expert_rows": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_vp, _c_vp, _c_i64, _c_vp, _c_vp, _c_i64, _c_f32, _c_f32, _c_vp, _c_vp, _c_i64,
                                      _c_i64, _c_i64, _c_vp]),
     "nvx_moe_order_max_experts": (_c_i64, []),
-    "nvx_moe_order": (_c_i32, [_c_vp, _c_i64, _c_i64, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp]),
-    "nvx_moe_expert_grouped_max_width": (_c_i64, []),
-    "nvx_moe_expert_grouped": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_vp, _c_i64, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_f32, _c_f32, _c_vp, _c_vp,
-                                        _c_i64, _c_i64, _c_i64, _c_vp]),
+    "nvx_moe_order": (_c_i32, [_c_vp, _c_i64, _c_i64, _c_vp, _c_vp, _c_vp]),
     "nvx_moe_scatter_rows": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_vp, _c_vp, _c_i64, _c_vp, _c_i64, _c_i64, _c_vp]),
     "nvx_moe_glu": (_c_i32, [_c_vp, _c_i32, _c_f32, _c_f32, _c_vp, _c_i64, _c_i64, _c_vp]),
     "nvx_moe_gather_rows": (_c_i32, [_c_vp, _c_i32, _c_vp, _c_i64, _c_vp, _c_i64, _c_i64, _c_vp]),

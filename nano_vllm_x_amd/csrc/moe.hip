@@ -115,109 +115,6 @@ __global__ __launch_bounds__(256) void moe_rows_down_kernel(const float* __restr
     }
 }
 
-// The same two steps with the pairs taken expert by expert (their order and the experts' offsets come from nvx_moe_order), so that
-// an expert's weights are read once for up to four of its pairs instead of once per pair: a workgroup takes 32 rows of ONE expert,
-// stages four pairs' inputs in LDS, and every weight it loads feeds four sums.  Pairs are addressed by their place in expert order:
-// y (places, ff) float32, out_pairs (places, width); the tokens' sums over their choices are nvx_moe_gather_rows' work.
-__device__ __forceinline__ float wave_sum_dpp(float v) {      // DPP within 16 lanes, lane-swap instructions across them
-    v = quarter_sum(v);
-    v += xor16(v);
-    v += xor32(v);
-    return v;
-}
-
-constexpr int MOE_PG = 4;         // pairs that share a pass over the weights
-
-template <typename A, bool VEC>
-__device__ __forceinline__ void lane_dot4(const A* __restrict__ wrow, const float* __restrict__ xs, int n, int lane, float acc[MOE_PG]) {
-#pragma unroll
-    for (int p = 0; p < MOE_PG; ++p) acc[p] = 0.f;
-    if constexpr (VEC) {
-        typedef A vec8 __attribute__((ext_vector_type(8)));
-        for (int c = lane * 8; c < n; c += 512) {
-            const vec8 v = *reinterpret_cast<const vec8*>(wrow + c);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const float wv = (float)v[i];
-#pragma unroll
-                for (int p = 0; p < MOE_PG; ++p) acc[p] += wv * xs[p * n + c + i];
-            }
-        }
-    } else {
-        for (int c = lane; c < n; c += 64) {
-            const float wv = ld_f(wrow, c);
-#pragma unroll
-            for (int p = 0; p < MOE_PG; ++p) acc[p] += wv * xs[p * n + c];
-        }
-    }
-}
-
-template <typename A, bool VEC>
-__global__ __launch_bounds__(256) void moe_grouped_up_kernel(const A* __restrict__ h, int64_t h_stride, const float* __restrict__ wts, int top,
-                                                            const int32_t* __restrict__ order, const int32_t* __restrict__ offsets,
-                                                            const A* __restrict__ w_gu, float limit, float alpha, float* __restrict__ y,
-                                                            int width, int ff) {
-    extern __shared__ float sm[];      // MOE_PG scaled inputs (width each)
-    const int e = blockIdx.y;
-    const int lo = offsets[e], hi = offsets[e + 1];
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const A* wg = w_gu + (int64_t)e * 2 * ff * width;
-    for (int p0 = lo; p0 < hi; p0 += MOE_PG) {
-        __syncthreads();
-        for (int i = threadIdx.x; i < MOE_PG * width; i += 256) {
-            const int p = i / width, c = i % width;
-            float v = 0.f;
-            if (p0 + p < hi) {
-                const int r = order[p0 + p];
-                v = (float)(A)(wts[r] * ld_f(h, (int64_t)(r / top) * h_stride + c));
-            }
-            sm[i] = v;
-        }
-        __syncthreads();
-        for (int i = 0; i < MOE_ROWS / 4; ++i) {
-            const int j = blockIdx.x * MOE_ROWS + wave * (MOE_ROWS / 4) + i;
-            if (j >= ff) break;
-            float g[MOE_PG], u[MOE_PG];
-            lane_dot4<A, VEC>(wg + (int64_t)j * width, sm, width, lane, g);
-            lane_dot4<A, VEC>(wg + (int64_t)(ff + j) * width, sm, width, lane, u);
-#pragma unroll
-            for (int p = 0; p < MOE_PG; ++p) {
-                const float gs = wave_sum_dpp(g[p]), us = wave_sum_dpp(u[p]);
-                if (lane == 0 && p0 + p < hi) y[(int64_t)(p0 + p) * ff + j] = (float)(A)glu_act((float)(A)gs, (float)(A)us, limit, alpha);
-            }
-        }
-    }
-}
-
-template <typename A, bool VEC>
-__global__ __launch_bounds__(256) void moe_grouped_down_kernel(const float* __restrict__ y, const int32_t* __restrict__ offsets,
-                                                              const A* __restrict__ w_d, A* __restrict__ out_pairs, int width, int ff) {
-    extern __shared__ float sm[];      // MOE_PG rows of hidden activations (ff each)
-    const int e = blockIdx.y;
-    const int lo = offsets[e], hi = offsets[e + 1];
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const A* wd = w_d + (int64_t)e * width * ff;
-    for (int p0 = lo; p0 < hi; p0 += MOE_PG) {
-        __syncthreads();
-        for (int i = threadIdx.x; i < MOE_PG * ff; i += 256) {
-            const int p = i / ff, j = i % ff;
-            sm[i] = p0 + p < hi ? y[(int64_t)(p0 + p) * ff + j] : 0.f;
-        }
-        __syncthreads();
-        for (int i = 0; i < MOE_ROWS / 4; ++i) {
-            const int c = blockIdx.x * MOE_ROWS + wave * (MOE_ROWS / 4) + i;
-            if (c >= width) break;
-            float o[MOE_PG];
-            lane_dot4<A, VEC>(wd + (int64_t)c * ff, sm, ff, lane, o);
-#pragma unroll
-            for (int p = 0; p < MOE_PG; ++p) {
-                const float os = wave_sum_dpp(o[p]);
-                if (lane == 0 && p0 + p < hi) st_f(out_pairs, (int64_t)(p0 + p) * width + c, os);
-            }
-        }
-    }
-}
-
 // xs[dst[r]] = wts[r] * h[r / top]  for every (token, choice) pair r: the experts' inputs in expert order
 template <typename A>
 __global__ __launch_bounds__(256) void moe_scatter_rows_kernel(const A* __restrict__ h, int64_t h_stride, const float* __restrict__ wts,
@@ -258,8 +155,7 @@ __global__ __launch_bounds__(256) void moe_gather_rows_kernel(const A* __restric
 // them per expert into LDS (cnt[e][thread]), the prefix sums over (expert, thread) give every thread its first position per
 // expert, and a second walk over the same run hands the positions out.  n_exp * 256 counters must fit LDS.
 __global__ __launch_bounds__(256) void moe_order_kernel(const int32_t* __restrict__ idx, int64_t n, int n_exp, int64_t* __restrict__ dst,
-                                                       int32_t* __restrict__ counts, int32_t* __restrict__ order,
-                                                       int32_t* __restrict__ offsets) {
+                                                       int32_t* __restrict__ counts) {
     extern __shared__ int cnt[];      // n_exp rows of 256, then n_exp bases
     int* base = cnt + n_exp * 256;
     const int tid = threadIdx.x;
@@ -279,22 +175,12 @@ __global__ __launch_bounds__(256) void moe_order_kernel(const int32_t* __restric
     __syncthreads();
     if (tid == 0) {
         int run = 0;
-        for (int e = 0; e < n_exp; ++e) {
-            const int c = base[e];
-            base[e] = run;
-            if (offsets) offsets[e] = run;
-            run += c;
-        }
-        if (offsets) offsets[n_exp] = run;
+        for (int e = 0; e < n_exp; ++e) { const int c = base[e]; base[e] = run; run += c; }
     }
     __syncthreads();
     for (int64_t r = lo; r < hi; ++r) {
         const int e = idx[r];
-        if (e >= 0 && e < n_exp) {
-            const int place = base[e] + cnt[e * 256 + tid]++;
-            dst[r] = place;
-            if (order) order[place] = (int32_t)r;
-        }
+        if (e >= 0 && e < n_exp) dst[r] = base[e] + cnt[e * 256 + tid]++;
     }
 }
 
@@ -304,13 +190,12 @@ using namespace NVX_NS;
 
 extern "C" int64_t nvx_moe_order_max_experts(void) { return (48 * 1024 / 4) / 257; }
 
-extern "C" int nvx_moe_order(const int32_t* idx, int64_t n, int64_t n_exp, int64_t* dst, int32_t* counts, int32_t* order, int32_t* offsets,
-                             nvx_stream_t stream) {
+extern "C" int nvx_moe_order(const int32_t* idx, int64_t n, int64_t n_exp, int64_t* dst, int32_t* counts, nvx_stream_t stream) {
     NVX_REQUIRE(n >= 0 && n < (1ll << 31) && n_exp > 0 && n_exp <= nvx_moe_order_max_experts(), NVX_EINVAL,
                 "nvx_moe_order: bad sizes (the experts' counters must fit LDS)");
     NVX_REQUIRE(idx && dst && counts, NVX_EINVAL, "nvx_moe_order: null pointer");
     hipLaunchKernelGGL(moe_order_kernel, dim3(1), dim3(256), (size_t)(n_exp * 257) * sizeof(int), (hipStream_t)stream, idx, n, (int)n_exp, dst,
-                       counts, order, offsets);
+                       counts);
     return nvx_check_launch("nvx_moe_order");
 }
 
@@ -358,44 +243,6 @@ extern "C" int nvx_moe_expert_rows(const void* h, int64_t h_stride, int fmt, con
     NVX_FMT_CALL(fmt, launch_moe_rows<A_>(h, h_stride, idx, wts, (int)top, w_gu, w_d, limit, alpha, ws, out, n_tok, (int)width, (int)ff,
                                           (hipStream_t)stream));
     return nvx_check_launch("nvx_moe_expert_rows");
-}
-
-template <typename A>
-static void launch_moe_grouped(const void* h, int64_t h_stride, const float* wts, int top, const int32_t* order, const int32_t* offsets,
-                               const void* w_gu, const void* w_d, int n_exp, float limit, float alpha, float* ws, void* out_pairs, int width, int ff,
-                               hipStream_t s) {
-    const bool vec = sizeof(A) == 2 && width % 8 == 0 && ff % 8 == 0 && nvx_aligned16(w_gu) && nvx_aligned16(w_d);
-    const dim3 up((unsigned)((ff + MOE_ROWS - 1) / MOE_ROWS), (unsigned)n_exp);
-    const dim3 down((unsigned)((width + MOE_ROWS - 1) / MOE_ROWS), (unsigned)n_exp);
-    const size_t lds_up = (size_t)MOE_PG * width * sizeof(float), lds_down = (size_t)MOE_PG * ff * sizeof(float);
-    if (vec) {
-        hipLaunchKernelGGL((moe_grouped_up_kernel<A, true>), up, dim3(256), lds_up, s, (const A*)h, h_stride, wts, top, order, offsets, (const A*)w_gu,
-                           limit, alpha, ws, width, ff);
-        hipLaunchKernelGGL((moe_grouped_down_kernel<A, true>), down, dim3(256), lds_down, s, (const float*)ws, offsets, (const A*)w_d,
-                           (A*)out_pairs, width, ff);
-    } else {
-        hipLaunchKernelGGL((moe_grouped_up_kernel<A, false>), up, dim3(256), lds_up, s, (const A*)h, h_stride, wts, top, order, offsets, (const A*)w_gu,
-                           limit, alpha, ws, width, ff);
-        hipLaunchKernelGGL((moe_grouped_down_kernel<A, false>), down, dim3(256), lds_down, s, (const float*)ws, offsets, (const A*)w_d,
-                           (A*)out_pairs, width, ff);
-    }
-}
-
-extern "C" int64_t nvx_moe_expert_grouped_max_width(void) { return 65536 / 4 / MOE_PG; }
-
-extern "C" int nvx_moe_expert_grouped(const void* h, int64_t h_stride, int fmt, const float* wts, int64_t top, const int32_t* order,
-                                      const int32_t* offsets, const void* w_gu, const void* w_d, int64_t n_exp, float limit, float alpha,
-                                      float* ws, void* out_pairs, int64_t n_tok, int64_t width, int64_t ff, nvx_stream_t stream) {
-    NVX_REQUIRE(fmt >= 0 && fmt <= 2, NVX_EINVAL, "nvx_moe_expert_grouped: fmt must be 0, 1 or 2");
-    NVX_REQUIRE(n_tok >= 0 && top > 0 && n_tok * top < (1ll << 31) && n_exp > 0 && n_exp <= 65535 && width > 0 && ff > 0 && h_stride >= width,
-                NVX_EINVAL, "nvx_moe_expert_grouped: bad sizes");
-    NVX_REQUIRE(width <= nvx_moe_expert_grouped_max_width() && ff <= nvx_moe_expert_grouped_max_width(), NVX_EUNSUPPORTED,
-                "nvx_moe_expert_grouped: four rows of the width or of the hidden size do not fit LDS");
-    if (n_tok == 0) return NVX_OK;
-    NVX_REQUIRE(h && wts && order && offsets && w_gu && w_d && ws && out_pairs, NVX_EINVAL, "nvx_moe_expert_grouped: null pointer");
-    NVX_FMT_CALL(fmt, launch_moe_grouped<A_>(h, h_stride, wts, (int)top, order, offsets, w_gu, w_d, (int)n_exp, limit, alpha, ws, out_pairs,
-                                             (int)width, (int)ff, (hipStream_t)stream));
-    return nvx_check_launch("nvx_moe_expert_grouped");
 }
 
 extern "C" int nvx_moe_scatter_rows(const void* h, int64_t h_stride, int fmt, const float* wts, const int64_t* dst, int64_t top, void* xs,

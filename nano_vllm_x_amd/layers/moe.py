@@ -33,14 +33,7 @@ class SigmoidInputMoE(nn.Module):
         idx, wts = ops.moe_route(ops.skinny_proj(h, self.router), self.top)
         if self._rows_fit is None:
             self._rows_fit = ops.moe_expert_rows_fits(self.width, self.ff)
-            self._grouped_fit = ops.moe_order_fits(self.experts) and ops.moe_expert_grouped_fits(self.width, self.ff)
         if self._rows_fit and (decode_step or t <= self.ROWS_PATH_TOKENS):
-            if self._grouped_fit and t * self.top > self.experts:
-                # more pairs than experts: some experts serve several pairs, so the pairs are taken expert by expert and an
-                # expert's weights are read once for up to four of them
-                dst, _, order, offsets = ops.moe_order(idx, self.experts, inverse=True)
-                pairs = ops.moe_expert_grouped(h, wts, order, offsets, self.w_gu, self.w_d, self.limit, self.alpha)
-                return ops.moe_gather_rows(pairs, dst)
             return ops.moe_expert_rows(h, idx, wts, self.w_gu, self.w_d, self.limit, self.alpha)
         if ops.moe_order_fits(self.experts):
             dst, counts = ops.moe_order(idx, self.experts)

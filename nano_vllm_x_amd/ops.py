@@ -1116,41 +1116,16 @@ def moe_order_fits(n_exp: int) -> bool:
     return n_exp <= _lib.load().nvx_moe_order_max_experts()
 
 
-def moe_order(idx, n_exp: int, inverse: bool = False):
+def moe_order(idx, n_exp: int):
     """idx (T, top) int32 expert ids -> (dst (T, top) int64, counts (n_exp) int32): dst[t][k] is the place of pair (t, k) when all
-    pairs are put in expert order (pairs of one expert keep their order), counts[e] the pairs of expert e.  `inverse`: also
-    (order (T * top) int32 with order[place] = pair, offsets (n_exp + 1) int32 with the first place of every expert)."""
+    pairs are put in expert order (pairs of one expert keep their order), counts[e] the pairs of expert e."""
     _dev(idx)
     _need(idx.dtype == torch.int32 and idx.is_contiguous() and idx.dim() == 2, "moe_order: idx must be contiguous int32 (T, top)")
     dst = torch.empty(idx.shape, dtype=torch.int64, device=idx.device)
     counts = torch.empty((n_exp,), dtype=torch.int32, device=idx.device)
-    order = torch.empty((idx.numel(),), dtype=torch.int32, device=idx.device) if inverse else None
-    offsets = torch.empty((n_exp + 1,), dtype=torch.int32, device=idx.device) if inverse else None
     lib = _lib.load()
-    _lib.check(lib.nvx_moe_order(_ptr(idx), idx.numel(), n_exp, _ptr(dst), _ptr(counts), _ptr(order), _ptr(offsets), _stream()), "nvx_moe_order")
-    return (dst, counts, order, offsets) if inverse else (dst, counts)
-
-
-def moe_expert_grouped_fits(width: int, ff: int) -> bool:
-    return max(width, ff) <= _lib.load().nvx_moe_expert_grouped_max_width()
-
-
-def moe_expert_grouped(h, wts, order, offsets, w_gu, w_d, limit: float, alpha: float):
-    """out_pairs[place] = expert(score * h[token]) for the pair at every place of the expert order (ops.moe_order with inverse),
-    an expert's weights read once for up to four of its pairs.  Returns (T * top, width); ops.moe_gather_rows(out_pairs, dst) sums
-    a token's choices."""
-    _dev(h, wts, order, offsets, w_gu, w_d)
-    n_exp, ff, width = _moe_weights(w_gu, w_d, "moe_expert_grouped")
-    t, top = wts.shape
-    _need(h.shape == (t, width) and h.stride(1) == 1 and h.dtype == w_gu.dtype, "moe_expert_grouped: h shape / format")
-    _need(wts.dtype == F32 and wts.is_contiguous() and order.dtype == torch.int32 and order.is_contiguous() and order.numel() == t * top and
-          offsets.dtype == torch.int32 and offsets.is_contiguous() and offsets.numel() == n_exp + 1, "moe_expert_grouped: order / offsets")
-    out = torch.empty((t * top, width), dtype=h.dtype, device=h.device)
-    ws = torch.empty((t * top, ff), dtype=F32, device=h.device)
-    lib = _lib.load()
-    _lib.check(lib.nvx_moe_expert_grouped(_ptr(h), h.stride(0), _fmt(h), _ptr(wts), top, _ptr(order), _ptr(offsets), _ptr(w_gu), _ptr(w_d), n_exp,
-                                          float(limit), float(alpha), _ptr(ws), _ptr(out), t, width, ff, _stream()), "nvx_moe_expert_grouped")
-    return out
+    _lib.check(lib.nvx_moe_order(_ptr(idx), idx.numel(), n_exp, _ptr(dst), _ptr(counts), _stream()), "nvx_moe_order")
+    return dst, counts
 
 
 def moe_scatter_rows(h, wts, dst):

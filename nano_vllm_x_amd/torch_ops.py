@@ -87,8 +87,6 @@ _DEFS = {
     "moe_route": "(Tensor logits, int top) -> (Tensor, Tensor)",
     "moe_expert_rows": "(Tensor h, Tensor idx, Tensor wts, Tensor w_gu, Tensor w_d, float limit, float alpha) -> Tensor",
     "moe_order": "(Tensor idx, int n_exp) -> (Tensor, Tensor)",
-    "moe_order_inverse": "(Tensor idx, int n_exp) -> (Tensor, Tensor, Tensor, Tensor)",
-    "moe_expert_grouped": "(Tensor h, Tensor wts, Tensor order, Tensor offsets, Tensor w_gu, Tensor w_d, float limit, float alpha) -> Tensor",
     "moe_scatter_rows": "(Tensor h, Tensor wts, Tensor dst) -> Tensor",
     "moe_glu": "(Tensor gu, float limit, float alpha) -> Tensor",
     "moe_gather_rows": "(Tensor ys, Tensor dst) -> Tensor",
@@ -301,14 +299,6 @@ def _moe_expert_rows(h, idx, wts, w_gu, w_d, limit, alpha):
 
 def _moe_order(idx, n_exp):
     return ops.moe_order(idx, n_exp)
-
-
-def _moe_order_inverse(idx, n_exp):
-    return ops.moe_order(idx, n_exp, inverse=True)
-
-
-def _moe_expert_grouped(h, wts, order, offsets, w_gu, w_d, limit, alpha):
-    return ops.moe_expert_grouped(h, wts, order, offsets, w_gu, w_d, limit, alpha)
 
 
 def _moe_scatter_rows(h, wts, dst):

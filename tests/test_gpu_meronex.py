@@ -298,9 +298,6 @@ def test_expert_order_is_a_stable_counting_sort(n_tok, top, experts):
     want[order] = torch.arange(order.numel())
     assert torch.equal(dst.cpu().view(-1), want) and torch.equal(counts.cpu().long(), torch.bincount(flat, minlength=experts))
     assert ops.moe_order_fits(47) and not ops.moe_order_fits(4000)
-    dst2, counts2, inv, offsets = ops.moe_order(idx.cuda(), experts, inverse=True)
-    assert torch.equal(dst2, dst) and torch.equal(counts2, counts) and torch.equal(inv.cpu().long(), order)
-    assert torch.equal(offsets.cpu().long(), torch.cat([torch.zeros(1, dtype=torch.long), torch.bincount(flat, minlength=experts).cumsum(0)]))
 
 
 @pytest.mark.parametrize("top,experts", [(1, 1), (1, 4), (2, 5), (3, 3)])
@@ -323,13 +320,9 @@ def test_experts_by_rows_and_by_expert_order_agree_with_the_restatement(top, exp
             moe.w_gu[e, ff:].copy_(p[f"e{e}.up"])
             moe.w_d[e].copy_(p[f"e{e}.down"])
         by_expert = moe(h.cuda()).cpu()                      # 45 tokens: per-expert matrix products
-        by_rows = moe(h.cuda(), decode_step=True).cpu()      # the same tokens as a decode step would take them (expert by expert)
-        from nano_vllm_x_amd import ops
-        idx, wts = ops.moe_route(ops.skinny_proj(h.cuda(), moe.router), top)
-        pair_by_pair = ops.moe_expert_rows(h.cuda(), idx, wts, moe.w_gu, moe.w_d, limit, 1.702).cpu()
+        by_rows = moe(h.cuda(), decode_step=True).cpu()      # the same tokens as a decode step would take them
     close(by_expert, want, 1e-5, "by expert")
     close(by_rows, want, 1e-5, "by rows")
-    close(pair_by_pair, want, 1e-5, "pair by pair")
     assert (want.abs() > 0).all()
 
 
