@@ -54,6 +54,53 @@ __device__ __forceinline__ float lane_dot(const A* __restrict__ wrow, const floa
     return acc;
 }
 
+// Two rows against one LDS vector, with the loads of four 512-element steps of both rows (eight 16-byte loads a lane) issued
+// before the first product: a wave alone then keeps 8 KB in flight instead of waiting out one load's latency per step.
+template <typename A, bool VEC>
+__device__ __forceinline__ void lane_dot2(const A* __restrict__ ra, const A* __restrict__ rb, const float* __restrict__ xs, int n, int lane,
+                                          float& out_a, float& out_b) {
+    float a = 0.f, b = 0.f;
+    if constexpr (VEC) {
+        typedef A vec8 __attribute__((ext_vector_type(8)));
+        int c = lane * 8;
+        for (; c + 1536 < n; c += 2048) {
+            vec8 va[4], vb[4];
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                va[s] = *reinterpret_cast<const vec8*>(ra + c + 512 * s);
+                vb[s] = *reinterpret_cast<const vec8*>(rb + c + 512 * s);
+            }
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const float x = xs[c + 512 * s + i];
+                    a += (float)va[s][i] * x;
+                    b += (float)vb[s][i] * x;
+                }
+            }
+        }
+        for (; c < n; c += 512) {
+            const vec8 va = *reinterpret_cast<const vec8*>(ra + c);
+            const vec8 vb = *reinterpret_cast<const vec8*>(rb + c);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float x = xs[c + i];
+                a += (float)va[i] * x;
+                b += (float)vb[i] * x;
+            }
+        }
+    } else {
+        for (int c = lane; c < n; c += 64) {
+            const float x = xs[c];
+            a += ld_f(ra, c) * x;
+            b += ld_f(rb, c) * x;
+        }
+    }
+    out_a = a;
+    out_b = b;
+}
+
 constexpr int MOE_ROWS = 32;      // weight rows per workgroup (8 per wave)
 
 template <typename A, bool VEC>
@@ -74,8 +121,7 @@ __global__ __launch_bounds__(256) void moe_rows_up_kernel(const A* __restrict__ 
     for (int i = 0; i < MOE_ROWS / 4; ++i) {         // all rows' loads in flight before the first reduction
         const int j = blockIdx.x * MOE_ROWS + wave * (MOE_ROWS / 4) + i;
         const int jc = j < ff ? j : ff - 1;
-        g[i] = lane_dot<A, VEC>(wg + (int64_t)jc * width, sm, width, lane);
-        u[i] = lane_dot<A, VEC>(wg + (int64_t)(ff + jc) * width, sm, width, lane);
+        lane_dot2<A, VEC>(wg + (int64_t)jc * width, wg + (int64_t)(ff + jc) * width, sm, width, lane, g[i], u[i]);
     }
 #pragma unroll
     for (int i = 0; i < MOE_ROWS / 4; ++i) {
@@ -101,9 +147,10 @@ __global__ __launch_bounds__(256) void moe_rows_down_kernel(const float* __restr
         const A* wd = w_d + (int64_t)idx[t * top + k] * width * ff;
         float part[MOE_ROWS / 4];
 #pragma unroll
-        for (int i = 0; i < MOE_ROWS / 4; ++i) {
+        for (int i = 0; i < MOE_ROWS / 4; i += 2) {
             const int c = blockIdx.x * MOE_ROWS + wave * (MOE_ROWS / 4) + i;
-            part[i] = lane_dot<A, VEC>(wd + (int64_t)(c < width ? c : width - 1) * ff, sm, ff, lane);
+            lane_dot2<A, VEC>(wd + (int64_t)(c < width ? c : width - 1) * ff, wd + (int64_t)(c + 1 < width ? c + 1 : width - 1) * ff, sm, ff, lane,
+                              part[i], part[i + 1]);
         }
 #pragma unroll
         for (int i = 0; i < MOE_ROWS / 4; ++i) o[i] += (float)(A)wave_sum(part[i]);
