@@ -235,7 +235,7 @@ __global__ __launch_bounds__(256) void moe_order_kernel(const int32_t* __restric
 
 using namespace NVX_NS;
 
-extern "C" int64_t nvx_moe_order_max_experts(void) { return (48 * 1024 / 4) / 257; }
+extern "C" int64_t nvx_moe_order_max_experts(void) { return (64 * 1024 / 4) / 257; }
 
 extern "C" int nvx_moe_order(const int32_t* idx, int64_t n, int64_t n_exp, int64_t* dst, int32_t* counts, nvx_stream_t stream) {
     NVX_REQUIRE(n >= 0 && n < (1ll << 31) && n_exp > 0 && n_exp <= nvx_moe_order_max_experts(), NVX_EINVAL,

@@ -33,18 +33,13 @@ class SigmoidInputMoE(nn.Module):
         idx, wts = ops.moe_route(ops.skinny_proj(h, self.router), self.top)
         if self._rows_fit is None:
             self._rows_fit = ops.moe_expert_rows_fits(self.width, self.ff)
-        if self._rows_fit and (decode_step or t <= self.ROWS_PATH_TOKENS):
+            self._order_fit = ops.moe_order_fits(self.experts)      # more experts than the ordering kernel holds: pair by pair
+            if not (self._rows_fit or self._order_fit):
+                raise NotImplementedError(f"{self.experts} experts of {self.ff} x {self.width}: neither expert path is built for these sizes")
+        if self._rows_fit and (decode_step or t <= self.ROWS_PATH_TOKENS or not self._order_fit):
             return ops.moe_expert_rows(h, idx, wts, self.w_gu, self.w_d, self.limit, self.alpha)
-        if ops.moe_order_fits(self.experts):
-            dst, counts = ops.moe_order(idx, self.experts)
-            counts = counts.tolist()
-        else:                                  # more experts than the ordering kernel's counters hold: a library sort
-            flat = idx.view(-1).long()
-            order = torch.argsort(flat, stable=True)
-            dst = torch.empty_like(order)
-            dst[order] = torch.arange(order.numel(), device=order.device)
-            dst = dst.view(t, self.top)
-            counts = torch.bincount(flat, minlength=self.experts).tolist()
+        dst, counts = ops.moe_order(idx, self.experts)
+        counts = counts.tolist()
         xs = ops.moe_scatter_rows(h, wts, dst)
         gu = torch.empty((xs.shape[0], 2 * self.ff), dtype=h.dtype, device=h.device)
         a = 0

@@ -259,7 +259,8 @@ def test_capped_attention_finds_one_key_among_hundreds(fmt, vdim):
     key is lost, the mask is off by one, or the cap is left out.  The last query sees itself; the one before must not see it."""
     from nano_vllm_x_amd import ops
     g = torch.Generator().manual_seed(vdim)
-    heads, kvh, dim, n, pool, cap, scale = 4, 2, 24, 700, 1024, 6.0, 0.5
+    heads, kvh, n, pool, cap, scale = 4, 2, 700, 1024, 6.0, 0.5
+    dim = 20 if vdim in (10, 64) else 24          # 20: no 16-byte loads of the key rows in the 16-bit format either
     k = 0.05 * torch.randn(n, kvh, dim, generator=g)
     v = torch.randn(n, kvh, vdim, generator=g)
     q = torch.randn(3, heads, dim, generator=g)          # queries of the last three tokens
@@ -286,7 +287,7 @@ def test_capped_attention_finds_one_key_among_hundreds(fmt, vdim):
     assert (out[1, 3] - out[2, 3]).abs().max() > 0.1          # the last query's own key changes head 3
 
 
-@pytest.mark.parametrize("n_tok,top,experts", [(20000, 2, 8), (5, 1, 1), (300, 3, 47), (257, 1, 2)])
+@pytest.mark.parametrize("n_tok,top,experts", [(20000, 2, 8), (5, 1, 1), (300, 3, 63), (257, 1, 2)])
 def test_expert_order_is_a_stable_counting_sort(n_tok, top, experts):
     from nano_vllm_x_amd import ops
     g = torch.Generator().manual_seed(n_tok)
@@ -297,7 +298,7 @@ def test_expert_order_is_a_stable_counting_sort(n_tok, top, experts):
     want = torch.empty_like(order)
     want[order] = torch.arange(order.numel())
     assert torch.equal(dst.cpu().view(-1), want) and torch.equal(counts.cpu().long(), torch.bincount(flat, minlength=experts))
-    assert ops.moe_order_fits(47) and not ops.moe_order_fits(4000)
+    assert ops.moe_order_fits(63) and not ops.moe_order_fits(4000)
 
 
 @pytest.mark.parametrize("top,experts", [(1, 1), (1, 4), (2, 5), (3, 3)])
