@@ -44,7 +44,7 @@ typedef void* nvx_stream_t;
  *   8: layers with a 32-bit residual stream and per-sequence state (`nvx_boundary_norm`, `nvx_canon_conv`, `nvx_relu2`,
  *      `nvx_mingru_scan`) and latent attention (`nvx_latent_prep`, `nvx_latent_attn`) added.
  *   9: nvx_boundary_norm can apply the convolution of a decode step in the same launch. */
-#define NVX_ABI_VERSION 14
+#define NVX_ABI_VERSION 15
 
 /* Library identification and diagnostics. */
 int nvx_abi_version(void);
@@ -527,7 +527,8 @@ int nvx_latent_attn(const void* q, const void* cache, int fmt, const int32_t* kv
  * nvx_softcap_attn:  token t of sequence b attends over the rows at slots kv_indices[kv_start[b] + j], j <= kv_len[b] - q_len[b] +
  *     (t - qo_indptr[b]):  s_j = scale * q . k_j,  s_j <- cap tanh(s_j / cap) (cap > 0),  out = softmax(s) V.  Query head h reads
  *     key/value head h / (heads / kv_heads).  q (n_tok, heads * dim), k_cache (slots, kv_heads * dim), v_cache (slots, kv_heads *
- *     vdim), out (n_tok, heads * vdim).
+ *     vdim), out (n_tok, heads * vdim).  n_split > 1 (for steps of few tokens): a (token, head)'s keys are dealt out over n_split
+ *     workgroups whose partial results go to `part` (n_tok * heads * n_split * (vdim + 2) floats) and are merged by a second launch.
  * nvx_moe_route:  idx[t][k], wts[t][k] = the expert with the k-th largest logit of token t (ties: the lower id) and the sigmoid
  *     of that logit.
  * Expert e:  g = min(W_gate x, limit), u = clamp(W_up x, -limit, limit), y = g sigmoid(alpha g) (u + 1), result W_down y, with
@@ -576,7 +577,7 @@ int nvx_rope_vnorm_store(const void* x, int64_t x_stride, int fmt, const int64_t
 int nvx_softcap_attn(const void* q, const void* k_cache, const void* v_cache, int fmt, const int32_t* kv_indices,
                      const int64_t* kv_start, const int32_t* kv_len, const int32_t* qo_indptr, const int32_t* tok_seq,
                      float scale, float cap, void* out, int64_t n_tok, int64_t heads, int64_t kv_heads, int64_t dim, int64_t vdim,
-                     nvx_stream_t stream);
+                     int n_split, float* part, nvx_stream_t stream);
 int nvx_moe_route(const float* logits, int64_t n_tok, int64_t n_exp, int64_t top, int32_t* idx, float* wts, nvx_stream_t stream);
 int64_t nvx_moe_expert_rows_max_width(int64_t ff);
 int nvx_moe_expert_rows(const void* h, int64_t h_stride, int fmt, const int32_t* idx, const float* wts, int64_t top,

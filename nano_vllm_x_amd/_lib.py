@@ -109,7 +109,7 @@ SIGNATURES = {
     "nvx_rope_vnorm_store": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_vp, _c_vp, _c_f32, _c_i32, _c_f32, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_i64,
                                       _c_i64, _c_i64, _c_i64, _c_i64, _c_vp]),
     "nvx_softcap_attn": (_c_i32, [_c_vp, _c_vp, _c_vp, _c_i32, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_f32, _c_f32, _c_vp, _c_i64, _c_i64, _c_i64,
-                                  _c_i64, _c_i64, _c_vp]),
+                                  _c_i64, _c_i64, _c_i32, _c_vp, _c_vp]),
     "nvx_moe_route": (_c_i32, [_c_vp, _c_i64, _c_i64, _c_i64, _c_vp, _c_vp, _c_vp]),
     "nvx_moe_expert_rows_max_width": (_c_i64, [_c_i64]),
     "nvx_moe_expert_rows": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_vp, _c_vp, _c_i64, _c_vp, _c_vp, _c_i64, _c_f32, _c_f32, _c_vp, _c_vp, _c_i64,

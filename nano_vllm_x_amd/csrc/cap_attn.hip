@@ -62,7 +62,8 @@ __global__ __launch_bounds__(256) void softcap_attn_kernel(const A* __restrict__
                                                           const int32_t* __restrict__ kv_indices, const int64_t* __restrict__ kv_start,
                                                           const int32_t* __restrict__ kv_len, const int32_t* __restrict__ qo_indptr,
                                                           const int32_t* __restrict__ tok_seq, float scale, float cap, A* __restrict__ out,
-                                                          int heads, int kv_heads, int dim, int vdim, int vec_v_ok) {
+                                                          int heads, int kv_heads, int dim, int vdim, int vec_v_ok, int n_split,
+                                                          float* __restrict__ part) {
     extern __shared__ float sm[];
     float* sq = sm;                   // dim
     float* sacc = sq + dim;           // 4 * vdim
@@ -86,7 +87,8 @@ __global__ __launch_bounds__(256) void softcap_attn_kernel(const A* __restrict__
     float acc8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     // value rows by 16-byte loads: vdim = 8 * (a power of two up to 64), rows 16-byte aligned (the caller checks the base)
     const bool vec_values = VEC && (vdim & 7) == 0 && ((vdim >> 3) & ((vdim >> 3) - 1)) == 0 && (vdim >> 3) <= 64 && vec_v_ok;
-    for (int j0 = wave * 64; j0 < visible; j0 += 256) {
+    // with n_split > 1 (steps of few tokens) the key tiles are dealt out over n_split workgroups as well as over the four waves
+    for (int j0 = (blockIdx.z * 4 + wave) * 64; j0 < visible; j0 += 256 * n_split) {
         const int j = j0 + lane;
         const bool valid = j < visible;
         const int slot = valid ? slots[j] : 0;
@@ -169,12 +171,37 @@ __global__ __launch_bounds__(256) void softcap_attn_kernel(const A* __restrict__
     const float mm = fmaxf(fmaxf(sml[0], sml[1]), fmaxf(sml[2], sml[3]));
     float f[4], total = 0.f;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) { f[w] = expf(sml[w] - mm); total += sml[4 + w] * f[w]; }
+    for (int w = 0; w < 4; ++w) { f[w] = sml[w] == -INFINITY ? 0.f : expf(sml[w] - mm); total += sml[4 + w] * f[w]; }
+    float* pr = n_split > 1 ? part + ((t * heads + hd) * (int64_t)n_split + blockIdx.z) * (vdim + 2) : nullptr;
     for (int e = threadIdx.x; e < vdim; e += 256) {
         float o = 0.f;
 #pragma unroll
         for (int w = 0; w < 4; ++w) o += sacc[w * vdim + e] * f[w];
-        st_f(out, t * (int64_t)heads * vdim + (int64_t)hd * vdim + e, o / total);
+        if (pr) pr[2 + e] = o;
+        else st_f(out, t * (int64_t)heads * vdim + (int64_t)hd * vdim + e, o / total);
+    }
+    if (pr && threadIdx.x == 0) { pr[0] = mm; pr[1] = total; }
+}
+
+// out = the n_split partial results of a (token, head) merged: each is (maximum, sum, unnormalised values); one wave each.
+template <typename A>
+__global__ __launch_bounds__(64) void softcap_merge_kernel(const float* __restrict__ part, int n_split, A* __restrict__ out, int vdim) {
+    const int64_t row = blockIdx.x;
+    const float* pr = part + row * n_split * (vdim + 2);
+    float mm = -INFINITY;
+    for (int s = 0; s < n_split; ++s) mm = fmaxf(mm, pr[s * (vdim + 2)]);
+    float total = 0.f;
+    for (int s = 0; s < n_split; ++s) {
+        const float m = pr[s * (vdim + 2)];
+        total += m == -INFINITY ? 0.f : pr[s * (vdim + 2) + 1] * expf(m - mm);
+    }
+    for (int e = threadIdx.x; e < vdim; e += 64) {
+        float o = 0.f;
+        for (int s = 0; s < n_split; ++s) {
+            const float m = pr[s * (vdim + 2)];
+            if (m != -INFINITY) o += pr[s * (vdim + 2) + 2 + e] * expf(m - mm);
+        }
+        st_f(out, row * vdim + e, o / total);
     }
 }
 
@@ -203,7 +230,7 @@ extern "C" int nvx_rope_vnorm_store(const void* x, int64_t x_stride, int fmt, co
 extern "C" int nvx_softcap_attn(const void* q, const void* k_cache, const void* v_cache, int fmt, const int32_t* kv_indices,
                                 const int64_t* kv_start, const int32_t* kv_len, const int32_t* qo_indptr, const int32_t* tok_seq,
                                 float scale, float cap, void* out, int64_t n_tok, int64_t heads, int64_t kv_heads, int64_t dim, int64_t vdim,
-                                nvx_stream_t stream) {
+                                int n_split, float* part, nvx_stream_t stream) {
     NVX_REQUIRE(fmt >= 0 && fmt <= 2, NVX_EINVAL, "nvx_softcap_attn: fmt must be 0, 1 or 2");
     NVX_REQUIRE(n_tok >= 0 && n_tok <= 65535 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && dim <= 4096 && vdim > 0 && vdim <= 512,
                 NVX_EINVAL, "nvx_softcap_attn: bad sizes (at most 65535 tokens a step, key size <= 4096, value size <= 512)");
@@ -211,12 +238,13 @@ extern "C" int nvx_softcap_attn(const void* q, const void* k_cache, const void* 
     NVX_REQUIRE(q && k_cache && v_cache && kv_indices && kv_start && kv_len && out, NVX_EINVAL, "nvx_softcap_attn: null pointer");
     NVX_REQUIRE((tok_seq != nullptr) == (qo_indptr != nullptr), NVX_EINVAL, "nvx_softcap_attn: tok_seq and qo_indptr go together");
     const size_t lds = (size_t)(dim + 4 * vdim + 8) * sizeof(float);
-    const dim3 grid((unsigned)heads, (unsigned)n_tok);
+    NVX_REQUIRE(n_split >= 1 && n_split <= 64 && (n_split == 1 || part), NVX_EINVAL, "nvx_softcap_attn: a key split needs its workspace");
+    const dim3 grid((unsigned)heads, (unsigned)n_tok, (unsigned)n_split);
 #define NVX_CAP_ATTN_V(EPL, VEC)                                                                                                          \
     NVX_FMT_CALL(fmt, hipLaunchKernelGGL((softcap_attn_kernel<A_, EPL, VEC && sizeof(A_) == 2>), grid, dim3(256), lds, (hipStream_t)stream,     \
                                          (const A_*)q, (const A_*)k_cache, (const A_*)v_cache, kv_indices, kv_start, kv_len, qo_indptr,      \
                                          tok_seq, scale, cap, (A_*)out, (int)heads, (int)kv_heads, (int)dim, (int)vdim,       \
-                                         (int)nvx_aligned16(v_cache)))
+                                         (int)nvx_aligned16(v_cache), n_split, part))
 #define NVX_CAP_ATTN(EPL) do { if (vec) NVX_CAP_ATTN_V(EPL, true); else NVX_CAP_ATTN_V(EPL, false); } while (0)
     const bool vec = fmt != 2 && dim % 8 == 0 && nvx_aligned16(k_cache);
     if (vdim <= 64) NVX_CAP_ATTN(1);
@@ -224,6 +252,9 @@ extern "C" int nvx_softcap_attn(const void* q, const void* k_cache, const void* 
     else if (vdim <= 256) NVX_CAP_ATTN(4);
     else NVX_CAP_ATTN(8);
 #undef NVX_CAP_ATTN_V
+    if (n_split > 1)
+        NVX_FMT_CALL(fmt, hipLaunchKernelGGL(softcap_merge_kernel<A_>, dim3((unsigned)(n_tok * heads)), dim3(64), 0, (hipStream_t)stream,
+                                             (const float*)part, n_split, (A_*)out, (int)vdim));
 #undef NVX_CAP_ATTN
     return nvx_check_launch("nvx_softcap_attn");
 }

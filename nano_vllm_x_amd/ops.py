@@ -8,6 +8,8 @@ capturable into a hipGraph.  `nano_vllm_x_amd.torch_ops` registers the stateless
 """
 from __future__ import annotations
 
+from typing import Optional
+
 import torch
 
 from . import _lib
@@ -1051,8 +1053,12 @@ def rope_vnorm_store(qkv, positions, freq, mag: float, rot_dims: int, eps: float
     return q
 
 
+SOFTCAP_SPLIT_BELOW = 1024      # (token, head) pairs of a step below which the keys are split over workgroups too
+SOFTCAP_SPLITS = 4
+
+
 def softcap_attn(q, k_cache, v_cache, kv_indices, kv_start, kv_len, layout: StepLayout, scale: float, cap: float, heads: int,
-                 kv_heads: int, dim: int, vdim: int):
+                 kv_heads: int, dim: int, vdim: int, n_split: Optional[int] = None):
     """Causal attention of q (T, heads * dim) over cached rows: sequence b's tokens are at slots kv_indices[kv_start[b] :
     kv_start[b] + kv_len[b]]; scores scale * q . k pass cap * tanh(. / cap) (cap <= 0: not) before the softmax.
     Returns (T, heads * vdim) in q's format."""
@@ -1066,10 +1072,15 @@ def softcap_attn(q, k_cache, v_cache, kv_indices, kv_start, kv_len, layout: Step
     _need(kv_start.dtype == torch.int64 and kv_start.numel() >= layout.n_seq, "softcap_attn: kv_start must be int64 (B)")
     _need(kv_len.dtype == torch.int32 and kv_len.numel() >= layout.n_seq, "softcap_attn: kv_len must be int32 (B)")
     out = torch.empty((t, heads * vdim), dtype=q.dtype, device=q.device)
+    # a step of few tokens is few workgroups, each walking all of its sequence's keys: their keys are dealt out over several
+    # workgroups whose partial results a second launch merges (the choice depends on the step's shape only, never on its data)
+    if n_split is None:
+        n_split = SOFTCAP_SPLITS if t * heads < SOFTCAP_SPLIT_BELOW else 1
+    part = torch.empty((t * heads * n_split * (vdim + 2),), dtype=F32, device=q.device) if n_split > 1 else None
     lib = _lib.load()
     _lib.check(lib.nvx_softcap_attn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _fmt(q), _ptr(kv_indices), _ptr(kv_start), _ptr(kv_len),
                                     _ptr(layout.qo_indptr), _ptr(layout.tok_seq), float(scale), float(cap), _ptr(out), t, heads, kv_heads, dim,
-                                    vdim, _stream()), "nvx_softcap_attn")
+                                    vdim, n_split, _ptr(part), _stream()), "nvx_softcap_attn")
     return out
 
 

@@ -271,8 +271,12 @@ def test_capped_attention_finds_one_key_among_hundreds(fmt, vdim):
     kc, vc = torch.zeros(pool, kvh * dim, dtype=fmt), torch.zeros(pool, kvh * vdim, dtype=fmt)
     kc[slots.long()], vc[slots.long()] = k.view(n, -1).to(fmt), v.view(n, -1).to(fmt)
     lay = _layout(ops, [3], [n - 3], [0])
-    out = ops.softcap_attn(q.view(3, -1).to(fmt).cuda(), kc.cuda(), vc.cuda(), slots.cuda(), torch.tensor([0]).cuda(),
-                           torch.tensor([n], dtype=torch.int32).cuda(), lay, scale, cap, heads, kvh, dim, vdim).float().cpu().view(3, heads, vdim)
+    args = (q.view(3, -1).to(fmt).cuda(), kc.cuda(), vc.cuda(), slots.cuda(), torch.tensor([0]).cuda(), torch.tensor([n], dtype=torch.int32).cuda(),
+            lay, scale, cap, heads, kvh, dim, vdim)
+    out = ops.softcap_attn(*args, n_split=1).float().cpu().view(3, heads, vdim)
+    for splits in (2, 4, 13):      # the keys dealt out over several workgroups and merged; 13: some workgroups get no key tile at all
+        again = ops.softcap_attn(*args, n_split=splits).float().cpu().view(3, heads, vdim)
+        assert torch.allclose(again, out, atol=1e-5 if fmt == torch.float32 else 2e-2), splits
     kf, vf, qf = k.to(fmt).double(), v.to(fmt).double(), q.to(fmt).double()
     for i in range(3):
         vis = n - 2 + i
