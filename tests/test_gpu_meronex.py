@@ -353,6 +353,23 @@ def test_each_mixer_alone_whole_cut_and_token_by_token(tmp_path, name):
     eng.shutdown()
 
 
+def test_attention_at_the_edges_of_its_key_tiles(tmp_path):
+    """The attention kernel takes keys in tiles of 64 dealt out over waves and, on small steps, over workgroups: prompts that end
+    one key before, at and after a tile's edge, decoded tokens that cross the edges at 64, 128 and 256 keys one by one, and a
+    portion that starts in the middle of a tile."""
+    cfg = make_cfg([PAR, PAR])
+    w = weights_of(cfg, 12)
+    eng = make_engine(model_dir(tmp_path, cfg, w), pool=1024)
+    toks = tokens(262, cfg["vocab"], 6)
+    want = mo.forward(cfg, w, toks)
+    for n in (63, 64, 65, 128, 129):
+        close(replay(eng, {f"p{n}": toks[:n]}, [[(f"p{n}", n)]])[f"p{n}"], want[:n], F32_TOL, f"prompt of {n}")
+    sched = [[("a", 62)]] + [[("a", 1)]] * 5 + [[("a", 30)], [("a", 29)]] + [[("a", 1)]] * 4 + [[("a", 123)]] + [[("a", 1)]] * 9
+    assert sum(n for step in sched for _, n in step) == 262
+    close(replay(eng, {"a": toks}, sched)["a"], want, F32_TOL, "edges crossed token by token")
+    eng.shutdown()
+
+
 # ---- the whole stack ------------------------------------------------------------------------------------------------------
 def test_batches_of_unequal_requests_in_a_small_pool(tmp_path):
     """Four live requests at most in a pool smaller than the sum of all: portions beside single tokens, a request that
